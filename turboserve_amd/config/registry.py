@@ -64,3 +64,8 @@ def _ensure_builtin() -> None:
         from turboserve_amd.models.kisadra import kisadra_plan
 
         register_architecture("Kisadra", KisadraConfig.from_dict, kisadra_plan)
+    if "Dovudra" not in ARCHITECTURES:
+        from turboserve_amd.config.dovudra_config import DovudraConfig
+        from turboserve_amd.models.dovudra import dovudra_plan
+
+        register_architecture("Dovudra", DovudraConfig.from_dict, dovudra_plan)

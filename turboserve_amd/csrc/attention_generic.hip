@@ -6,7 +6,9 @@
 // otherwise (src/turboserve/engine/model/attention.py:139-148: keys <= ctx - q_len + j; the
 // window bound is this engine's); with chunk > 0 also lo >= (p / chunk) * chunk: a token sees its
 // own chunk of positions only, chunks counted from position 0 of the request.  sinks > 0 adds that
-// many keys of score 0 without a value to the softmax's denominator.  Without value pages the
+// many keys of score 0 without a value to the softmax's denominator; with sink_scores [Hq] their score
+// is the head's entry instead of 0 (it is not scaled and gets no bias).  distance_bias [Hq, L] (32-bit)
+// adds distance_bias[h][min(p - key, L - 1)] to the score of a key, after scale and cap.  Without value pages the
 // values are the first vdim elements of the keys themselves (a mixer that caches one vector per
 // token).  Keys and values are read through the request's block table
 // from key pages [NB, Hkv, BS, D] and transposed value pages [NB, Hkv, Dv, BS] (values may be wider
@@ -31,7 +33,9 @@ paged_attention_generic_kernel(T* __restrict__ out, const T* __restrict__ q, lon
                                const int* __restrict__ block_table, int table_width,
                                const int* __restrict__ token_seq, const int* __restrict__ positions,
                                int heads, int kv_heads, int dim, int vdim, int block_size, float scale,
-                               float softcap, int window, const float* __restrict__ slopes, int chunk, float sinks) {
+                               float softcap, int window, const float* __restrict__ slopes, int chunk, float sinks,
+                               const float* __restrict__ sink_scores, const float* __restrict__ distance_bias,
+                               int bias_len) {
   __shared__ float qs[ATTN_MAX_DIM];
   __shared__ float ps[ATTN_TILE];
   __shared__ long long rows[ATTN_TILE];  // per key of the tile: offset of its value column
@@ -50,6 +54,7 @@ paged_attention_generic_kernel(T* __restrict__ out, const T* __restrict__ q, lon
   const int* table = block_table + (size_t)seq * table_width;
   // A position encoding may bias the scores by the distance: + slope[h] * (key - p), in 32-bit.
   const float slope = slopes ? slopes[h] : 0.f;
+  const float* bias_row = distance_bias ? distance_bias + (size_t)h * bias_len : nullptr;
 
   const T* qrow = q + (size_t)t * q_stride + (size_t)h * dim;
   for (int d = lane; d < dim; d += ATTN_TILE) qs[d] = to_float(qrow[d]) * scale;
@@ -60,7 +65,7 @@ paged_attention_generic_kernel(T* __restrict__ out, const T* __restrict__ q, lon
 #pragma unroll
   for (int c = 0; c < CHUNKS; ++c) acc[c] = 0.f;
   // A sink is a key of score 0 that is always there: the running maximum starts at its score.
-  float m_run = sinks > 0.f ? 0.f : -INFINITY;
+  float m_run = sinks > 0.f ? (sink_scores ? sink_scores[h] : 0.f) : -INFINITY;
   float l_run = sinks > 0.f ? sinks : 0.f;
 
   for (int base = lo; base <= p; base += ATTN_TILE) {
@@ -78,6 +83,7 @@ paged_attention_generic_kernel(T* __restrict__ out, const T* __restrict__ q, lon
       for (int d = 0; d < dim; ++d) s = fmaf(qs[d], to_float(krow[d]), s);
       if (softcap > 0.f) s = softcap * tanhf(s / softcap);
       score = slopes ? fmaf(slope, (float)(key - p), s) : s;
+      if (bias_row) score += bias_row[min(p - key, bias_len - 1)];
     }
     const float m_new = fmaxf(m_run, wave_max(score));
     const float alpha = expf(m_run - m_new);  // 0 on the first tile (m_run = -inf, m_new finite)
@@ -113,24 +119,27 @@ paged_attention_generic_kernel(T* __restrict__ out, const T* __restrict__ q, lon
 // out [T, Hq, Dv] contiguous; q rows are q_stride elements apart (the fused projection output).
 // slopes [Hq] (32-bit) or null: the score of key j for the query at position p gets
 // slopes[h] * (j - p) added.  v_pages null: the values are the keys' first vdim elements.
+// sink_scores [Hq] (32-bit) or null; distance_bias [Hq, bias_len] (32-bit) or null.
 extern "C" int ts_paged_attention_generic(void* out, const void* q, long q_stride,
                                           const void* k_pages, const void* v_pages,
                                           const int* block_table, int table_width,
                                           const int* token_seq, const int* positions, int tokens,
                                           int heads, int kv_heads, int dim, int vdim, int block_size,
                                           float scale, float softcap, int window, const float* slopes, int chunk,
-                                          float sinks, int dtype, hipStream_t stream) {
+                                          float sinks, const float* sink_scores, const float* distance_bias,
+                                          int bias_len, int dtype, hipStream_t stream) {
   if (tokens == 0) return TS_OK;
   if (!out || !q || !k_pages || !block_table || !token_seq || !positions) return TS_ERR_ARG;
   if (chunk < 0 || !(sinks >= 0.f) || (!v_pages && vdim > dim)) return TS_ERR_ARG;
+  if ((sink_scores && !(sinks > 0.f)) || (distance_bias && bias_len < 1)) return TS_ERR_ARG;
   if (heads < 1 || kv_heads < 1 || heads % kv_heads != 0 || heads > 65535) return TS_ERR_SHAPE;
   if (dim < 1 || dim > ATTN_MAX_DIM || vdim < 1 || vdim > ATTN_MAX_DIM || block_size < 1 || table_width < 1)
     return TS_ERR_SHAPE;
   dim3 grid(tokens, heads), block(ATTN_TILE);
   if (dtype == TS_F32)
-    hipLaunchKernelGGL(paged_attention_generic_kernel<float>, grid, block, 0, stream, (float*)out, (const float*)q, q_stride, (const float*)k_pages, (const float*)v_pages, block_table, table_width, token_seq, positions, heads, kv_heads, dim, vdim, block_size, scale, softcap, window, slopes, chunk, sinks);
+    hipLaunchKernelGGL(paged_attention_generic_kernel<float>, grid, block, 0, stream, (float*)out, (const float*)q, q_stride, (const float*)k_pages, (const float*)v_pages, block_table, table_width, token_seq, positions, heads, kv_heads, dim, vdim, block_size, scale, softcap, window, slopes, chunk, sinks, sink_scores, distance_bias, bias_len);
   else if (dtype == TS_BF16)
-    hipLaunchKernelGGL(paged_attention_generic_kernel<bf16_t>, grid, block, 0, stream, (bf16_t*)out, (const bf16_t*)q, q_stride, (const bf16_t*)k_pages, (const bf16_t*)v_pages, block_table, table_width, token_seq, positions, heads, kv_heads, dim, vdim, block_size, scale, softcap, window, slopes, chunk, sinks);
+    hipLaunchKernelGGL(paged_attention_generic_kernel<bf16_t>, grid, block, 0, stream, (bf16_t*)out, (const bf16_t*)q, q_stride, (const bf16_t*)k_pages, (const bf16_t*)v_pages, block_table, table_width, token_seq, positions, heads, kv_heads, dim, vdim, block_size, scale, softcap, window, slopes, chunk, sinks, sink_scores, distance_bias, bias_len);
   else
     return TS_ERR_DTYPE;
   return ts_launch_status();

@@ -1,8 +1,8 @@
 // Paged attention on the matrix cores for the score rules and cache shapes the head-size-specialised
 // kernels do not take (bfloat16): keys and values of different widths, values that are the first
 // elements of the key rows themselves (a layer that caches one vector per token), a bias on the
-// scores that is linear in the distance, chunks of positions, a window, sinks in the softmax's
-// denominator.  Same arithmetic as ts_paged_attention_generic: scores, bias, masks and softmax in
+// scores that is linear in the distance or read from a table by the distance, chunks of positions, a
+// window, sinks in the softmax's denominator (of score 0, or of a score per head).  Same arithmetic as ts_paged_attention_generic: scores, bias, masks and softmax in
 // 32-bit; products of bfloat16 operands accumulated in 32-bit.
 //
 // A workgroup of four wavefronts owns 64 query rows and walks the keys they may see in tiles of 64:
@@ -69,7 +69,8 @@ attention_tiles_kernel(uint16_t* __restrict__ out, float* __restrict__ partial_o
                        const uint16_t* __restrict__ v_pages, const int* __restrict__ block_table, int table_width,
                        const int* __restrict__ query_start_loc, const int* __restrict__ context_lens,
                        const int* __restrict__ tiles, int first_seq, int heads, int kv_heads, int dk, int dv,
-                       int block_size, const float* __restrict__ slopes, FaRule rule, int splits) {
+                       int block_size, const float* __restrict__ slopes, FaRule rule, int splits,
+                       const float* __restrict__ sink_scores, const float* __restrict__ distance_bias, int bias_len) {
   extern __shared__ __attribute__((aligned(16))) uint16_t fa_lds[];
   constexpr int K_ROW = KD * 32 + FA_PAD;       // elements of a staged key row
   constexpr int V_ROW = FA_KEYS + FA_PAD;       // elements of a staged value column (64 keys)
@@ -135,7 +136,8 @@ attention_tiles_kernel(uint16_t* __restrict__ out, float* __restrict__ partial_o
   }
   // Per accumulator row i of this lane (row wave * 16 + 4 group + i): position, lowest key, slope.
   int pos[4], low[4];
-  float slope[4];
+  float slope[4], sink_at[4];
+  const float* bias_row[4];
 #pragma unroll
   for (int i = 0; i < 4; ++i) {
     const int r = wave * 16 + 4 * group + i;
@@ -143,6 +145,9 @@ attention_tiles_kernel(uint16_t* __restrict__ out, float* __restrict__ partial_o
     pos[i] = live ? row_position(r) : -1;  // an idle row sees nothing
     low[i] = live ? fa_lowest(pos[i], rule.window, rule.chunk) : 0;
     slope[i] = (slopes && live) ? slopes[row_head(r)] : 0.f;
+    // The row's line of the bias table (read by distance); an idle row reads head 0's and is masked.
+    bias_row[i] = distance_bias ? distance_bias + (size_t)(live ? row_head(r) : 0) * bias_len : nullptr;
+    sink_at[i] = (sink_scores && live) ? sink_scores[row_head(r)] : 0.f;
   }
   fa_f32x4 o[VD];
 #pragma unroll
@@ -153,7 +158,7 @@ attention_tiles_kernel(uint16_t* __restrict__ out, float* __restrict__ partial_o
   const bool own_sinks = rule.sinks > 0.f && splits == 1;
 #pragma unroll
   for (int i = 0; i < 4; ++i) {
-    m_run[i] = own_sinks ? 0.f : -INFINITY;
+    m_run[i] = own_sinks ? sink_at[i] : -INFINITY;
     l_run[i] = own_sinks ? rule.sinks : 0.f;
   }
 
@@ -272,7 +277,9 @@ attention_tiles_kernel(uint16_t* __restrict__ out, float* __restrict__ partial_o
 #pragma unroll
       for (int i = 0; i < 4; ++i) {
         float v = fmaf(slope[i], (float)(key - pos[i]), s[ct][i] * rule.scale);
-        v = (key >= low[i] && key <= pos[i]) ? v : -INFINITY;
+        const bool seen = key >= low[i] && key <= pos[i];
+        if (distance_bias) v += bias_row[i][seen ? min(pos[i] - key, bias_len - 1) : 0];
+        v = seen ? v : -INFINITY;
         s[ct][i] = v;
         tile_max[i] = fmaxf(tile_max[i], v);
       }
@@ -353,7 +360,8 @@ attention_tiles_kernel(uint16_t* __restrict__ out, float* __restrict__ partial_o
 __global__ void __launch_bounds__(128)
 attention_tiles_combine_kernel(uint16_t* __restrict__ out, const float* __restrict__ partial_o,
                                const float* __restrict__ partial_ml, const int* __restrict__ query_start_loc,
-                               int first_seq, int heads, int dv, int splits, float sinks) {
+                               int first_seq, int heads, int dv, int splits, float sinks,
+                               const float* __restrict__ sink_scores) {
   __shared__ float weight[FA_MAX_SPLITS];
   __shared__ float scratch[16];
   const int item = blockIdx.x, h = blockIdx.y;
@@ -361,10 +369,11 @@ attention_tiles_combine_kernel(uint16_t* __restrict__ out, const float* __restri
   const int sp = threadIdx.x;
   const float ms = sp < splits ? partial_ml[2 * (base + sp)] : -INFINITY;
   const float ls = sp < splits ? partial_ml[2 * (base + sp) + 1] : 0.f;
-  const float m = fmaxf(block_max(ms, scratch), sinks > 0.f ? 0.f : -INFINITY);
+  const float sink_at = sink_scores ? sink_scores[h] : 0.f;
+  const float m = fmaxf(block_max(ms, scratch), sinks > 0.f ? sink_at : -INFINITY);
   const float w = ms == -INFINITY ? 0.f : expf(ms - m);
   if (sp < splits) weight[sp] = w;
-  const float l = block_sum(ls * w, scratch) + (sinks > 0.f ? sinks * expf(0.f - m) : 0.f);  // (its barriers publish the weights)
+  const float l = block_sum(ls * w, scratch) + (sinks > 0.f ? sinks * expf(sink_at - m) : 0.f);  // (its barriers publish the weights)
   const float inv = l > 0.f ? 1.f / l : 0.f;
   const int row = query_start_loc[first_seq + item];
   for (int d = threadIdx.x; d < dv; d += blockDim.x) {
@@ -386,7 +395,8 @@ static int tiles_launch(bool single, bool values_in_keys, dim3 grid, hipStream_t
                         float* partial_ml, const uint16_t* q, long q_stride, const uint16_t* k_pages,
                         const uint16_t* v_pages, const int* block_table, int table_width, const int* query_start_loc,
                         const int* context_lens, const int* tiles, int first_seq, int heads, int kv_heads, int dk, int dv,
-                        int block_size, const float* slopes, FaRule rule, int splits) {
+                        int block_size, const float* slopes, FaRule rule, int splits, const float* sink_scores,
+                        const float* distance_bias, int bias_len) {
   constexpr size_t lds = (size_t)(FA_KEYS * (KD * 32 + FA_PAD) + VD * 16 * (FA_KEYS + FA_PAD) + 4 * 16 * (FA_KEYS + FA_PAD)) * sizeof(uint16_t);
   static_assert(lds <= 160 * 1024, "the staged tiles must fit in LDS");
 #define FA_GO(SINGLE, INKEYS)                                                                                          \
@@ -400,7 +410,8 @@ static int tiles_launch(bool single, bool values_in_keys, dim3 grid, hipStream_t
     }                                                                                                                  \
     hipLaunchKernelGGL((attention_tiles_kernel<KD, VD, SINGLE, INKEYS>), grid, dim3(FA_THREADS), lds, stream, out,     \
                        partial_o, partial_ml, q, q_stride, k_pages, v_pages, block_table, table_width, query_start_loc, \
-                       context_lens, tiles, first_seq, heads, kv_heads, dk, dv, block_size, slopes, rule, splits);     \
+                       context_lens, tiles, first_seq, heads, kv_heads, dk, dv, block_size, slopes, rule, splits,      \
+                       sink_scores, distance_bias, bias_len);                                                          \
   } while (0)
   if (single && values_in_keys) FA_GO(true, true);
   else if (single) FA_GO(true, false);
@@ -413,17 +424,21 @@ static int tiles_launch(bool single, bool values_in_keys, dim3 grid, hipStream_t
 // mode 0: prompt portions, `items` tiles (pairs: request, first row), each for every head;
 // mode 1: `items` requests of one token each from `first_seq` on, their keys shared out over `splits`.
 // out [T, heads, Dv] bfloat16.  v_pages null: the values are the keys' first Dv elements.
+// sink_scores [heads] (32-bit) or null: the score of the sinks, 0 without; distance_bias [heads, bias_len]
+// (32-bit) or null: the score of a key at distance n gets distance_bias[h][min(n, bias_len - 1)] added.
 extern "C" int ts_attention_tiles(void* out, void* partial_o, void* partial_ml, const void* q, long q_stride,
                                   const void* k_pages, const void* v_pages, const int* block_table, int table_width,
                                   const int* query_start_loc, const int* context_lens, const int* tiles, int items,
                                   int first_seq, int heads, int kv_heads, int dk, int dv, int block_size, float scale,
                                   float softcap, int window, int chunk, float sinks, const float* slopes, int mode,
-                                  int splits, hipStream_t stream) {
+                                  int splits, const float* sink_scores, const float* distance_bias, int bias_len,
+                                  hipStream_t stream) {
   if (items == 0) return TS_OK;
   if (!out || !q || !k_pages || !block_table || !query_start_loc || !context_lens) return TS_ERR_ARG;
   if (mode == 0 && (!tiles || splits != 1)) return TS_ERR_ARG;
   if (mode == 1 && splits > 1 && (!partial_o || !partial_ml)) return TS_ERR_ARG;
   if (mode < 0 || mode > 1 || splits < 1 || splits > FA_MAX_SPLITS) return TS_ERR_ARG;
+  if ((sink_scores && !(sinks > 0.f)) || (distance_bias && bias_len < 1)) return TS_ERR_ARG;
   if (heads < 1 || kv_heads < 1 || heads % kv_heads != 0 || heads > 65535) return TS_ERR_SHAPE;
   if (dk < 8 || dk > 448 || dk % 8 != 0 || dv < 8 || dv > 384 || dv % 8 != 0 || block_size < 8 || block_size % 8 != 0)
     return TS_ERR_SHAPE;
@@ -441,7 +456,7 @@ extern "C" int ts_attention_tiles(void* out, void* partial_o, void* partial_ml, 
   return tiles_launch<KD, VD>(single, in_keys, grid, stream, (uint16_t*)out, (float*)partial_o, (float*)partial_ml,     \
                               (const uint16_t*)q, q_stride, (const uint16_t*)k_pages, (const uint16_t*)v_pages,         \
                               block_table, table_width, query_start_loc, context_lens, tiles, first_seq, heads, kv_heads, \
-                              dk, dv, block_size, slopes, rule, splits)
+                              dk, dv, block_size, slopes, rule, splits, sink_scores, distance_bias, bias_len)
   if (kd <= 2 && vd <= 4) FA_SIZE(2, 4);
   if (kd <= 4 && vd <= 8) FA_SIZE(4, 8);
   if (kd <= 4 && vd <= 16) FA_SIZE(4, 16);
@@ -456,11 +471,11 @@ extern "C" int ts_attention_tiles(void* out, void* partial_o, void* partial_ml, 
 
 extern "C" int ts_attention_tiles_combine(void* out, const void* partial_o, const void* partial_ml,
                                           const int* query_start_loc, int items, int first_seq, int heads, int dv,
-                                          int splits, float sinks, hipStream_t stream) {
+                                          int splits, float sinks, const float* sink_scores, hipStream_t stream) {
   if (items == 0) return TS_OK;
   if (!out || !partial_o || !partial_ml || !query_start_loc || splits < 1 || splits > FA_MAX_SPLITS || heads < 1 || heads > 65535 || dv < 1)
     return TS_ERR_ARG;
   hipLaunchKernelGGL(attention_tiles_combine_kernel, dim3(items, heads), dim3(128), 0, stream, (uint16_t*)out,
-                     (const float*)partial_o, (const float*)partial_ml, query_start_loc, first_seq, heads, dv, splits, sinks);
+                     (const float*)partial_o, (const float*)partial_ml, query_start_loc, first_seq, heads, dv, splits, sinks, sink_scores);
   return ts_launch_status();
 }

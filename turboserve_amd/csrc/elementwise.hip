@@ -94,17 +94,52 @@ __device__ __forceinline__ float add_splits(const P* p, int splits, size_t strid
 
 // P is the type of `pending`: T, or float for `splits` partial sums of a product that are
 // `split_stride` elements apart and are added up here.
+// A pending output may carry a norm of its own (`post`): it is then divided by its root mean square,
+// multiplied by `post.gain` and by `post.scale`, all in 32-bit, before it is added (a block that
+// normalises a part's output before the residual sum).  `also` does not go with it.
+template <typename T>
+struct PostNorm {
+  const T* gain;  // null: the pending output is added as it is
+  float eps;
+  float scale;
+};
+
 template <typename T, typename P>
 __global__ void add_rmsnorm_kernel(T* __restrict__ y, float* __restrict__ residual,
                                    const P* __restrict__ pending, int splits, size_t split_stride,
                                    const T* __restrict__ w, const int* __restrict__ rows, float eps,
                                    int hidden, float gain_offset, int one_rounding,
-                                   const float* __restrict__ also, int also_splits, size_t also_stride) {
+                                   const float* __restrict__ also, int also_splits, size_t also_stride,
+                                   PostNorm<T> post) {
   __shared__ float scratch[16];
   const int src = rows ? rows[blockIdx.x] : blockIdx.x;
   const size_t in_base = (size_t)src * hidden;
   const size_t out_base = (size_t)blockIdx.x * hidden;
   float ss = 0.f;
+  if (post.gain) {
+    float pss = 0.f;
+    for (int i = threadIdx.x; i < hidden; i += blockDim.x) {
+      const float v = add_splits(pending + in_base + i, splits, split_stride, 0.f);
+      pss += v * v;
+    }
+    pss = block_sum(pss, scratch);
+    const float by = rsqrtf(pss / (float)hidden + post.eps) * post.scale;
+    // Without `rows` the sum is left in the residual stream; with `rows` it is formed again below.
+    for (int i = threadIdx.x; i < hidden; i += blockDim.x) {
+      const float v = add_splits(pending + in_base + i, splits, split_stride, 0.f);
+      const float s = residual[in_base + i] + v * by * to_float(post.gain[i]);
+      if (!rows) residual[in_base + i] = s;
+      ss += s * s;
+    }
+    ss = block_sum(ss, scratch);
+    const float rstd = rsqrtf(ss / (float)hidden + eps);
+    for (int i = threadIdx.x; i < hidden; i += blockDim.x) {
+      float s = residual[in_base + i];
+      if (rows) s += add_splits(pending + in_base + i, splits, split_stride, 0.f) * by * to_float(post.gain[i]);
+      y[out_base + i] = from_float<T>(with_gain<T>(s * rstd, to_float(w[i]), gain_offset, one_rounding));
+    }
+    return;
+  }
   for (int i = threadIdx.x; i < hidden; i += blockDim.x) {
     float s = residual[in_base + i];
     if (pending) s = add_splits(pending + in_base + i, splits, split_stride, s);
@@ -204,12 +239,13 @@ __device__ __forceinline__ void add_splits4(const P* p, int splits, size_t strid
 
 #define NORM_ITEMS 4
 
-template <typename T, typename P>
+template <typename T, typename P, bool POST>
 __global__ void add_rmsnorm_vec4_kernel(T* __restrict__ y, float* __restrict__ residual,
                                         const P* __restrict__ pending, int splits, size_t split_stride,
                                         const T* __restrict__ w, const int* __restrict__ rows, float eps,
                                         int hidden, float gain_offset, int one_rounding,
-                                        const float* __restrict__ also, int also_splits, size_t also_stride) {
+                                        const float* __restrict__ also, int also_splits, size_t also_stride,
+                                        PostNorm<T> post) {
   __shared__ float scratch[16];
   const int src = rows ? rows[blockIdx.x] : blockIdx.x;
   const size_t in_base = (size_t)src * hidden;
@@ -217,10 +253,43 @@ __global__ void add_rmsnorm_vec4_kernel(T* __restrict__ y, float* __restrict__ r
   const int quads = hidden / 4;
   float s[NORM_ITEMS][4], g[NORM_ITEMS][4];
   float ss = 0.f;
+  if (POST) {
+    // The pending output with its own norm: its sum of squares first, then the residual sum.
+    float p[NORM_ITEMS][4], pg[NORM_ITEMS][4];
+    float pss = 0.f;
+#pragma unroll
+    for (int it = 0; it < NORM_ITEMS; ++it) {
+      const int qd = threadIdx.x + it * blockDim.x;
+      if (qd < quads) {
+        Vec4Of<float>::load(residual + in_base + 4 * qd, s[it]);
+        Vec4Of<T>::load(w + 4 * qd, g[it]);
+        Vec4Of<T>::load(post.gain + 4 * qd, pg[it]);
+#pragma unroll
+        for (int e = 0; e < 4; ++e) p[it][e] = 0.f;
+        add_splits4(pending + in_base + 4 * qd, splits, split_stride, p[it]);
+#pragma unroll
+        for (int e = 0; e < 4; ++e) pss += p[it][e] * p[it][e];
+      }
+    }
+    pss = block_sum(pss, scratch);
+    const float by = rsqrtf(pss / (float)hidden + post.eps) * post.scale;
+#pragma unroll
+    for (int it = 0; it < NORM_ITEMS; ++it) {
+      const int qd = threadIdx.x + it * blockDim.x;
+      if (qd < quads) {
+#pragma unroll
+        for (int e = 0; e < 4; ++e) {
+          s[it][e] += p[it][e] * by * pg[it][e];
+          ss += s[it][e] * s[it][e];
+        }
+        if (!rows) Vec4Of<float>::store(residual + in_base + 4 * qd, s[it]);
+      }
+    }
+  }
 #pragma unroll
   for (int it = 0; it < NORM_ITEMS; ++it) {
     const int qd = threadIdx.x + it * blockDim.x;
-    if (qd < quads) {
+    if (!POST && qd < quads) {
       Vec4Of<float>::load(residual + in_base + 4 * qd, s[it]);
       Vec4Of<T>::load(w + 4 * qd, g[it]);  // with the other loads, not behind the reduction's barriers
       if (pending) add_splits4(pending + in_base + 4 * qd, splits, split_stride, s[it]);
@@ -248,38 +317,48 @@ template <typename T, typename P>
 static void launch_add_rmsnorm(void* y, float* residual, const void* pending, int splits, long split_stride,
                                const void* w, const int* rows, float eps, int out_rows, int hidden,
                                float gain_offset, int one_rounding, const float* also, int also_splits,
-                               long also_stride, hipStream_t stream) {
+                               long also_stride, const void* post_gain, float post_eps, float post_scale,
+                               hipStream_t stream) {
   // Few rows (decode): one large block per row; many rows (prefill): just enough threads.
   int threads = out_rows <= 256 ? 1024 : 256;
   const int need = (hidden / 4 + NORM_ITEMS - 1) / NORM_ITEMS;
   if (threads < need) threads = ((need + 63) / 64) * 64;
-  if (hidden % 4 == 0 && threads <= 1024) {
-    hipLaunchKernelGGL((add_rmsnorm_vec4_kernel<T, P>), dim3(out_rows), dim3(threads), 0, stream, (T*)y, residual,
+  const PostNorm<T> post = {(const T*)post_gain, post_eps, post_scale};
+  if (hidden % 4 == 0 && threads <= 1024 && post_gain) {
+    hipLaunchKernelGGL((add_rmsnorm_vec4_kernel<T, P, true>), dim3(out_rows), dim3(threads), 0, stream, (T*)y, residual,
                        (const P*)pending, splits, (size_t)split_stride, (const T*)w, rows, eps, hidden, gain_offset,
-                       one_rounding, also, also_splits, (size_t)also_stride);
+                       one_rounding, also, also_splits, (size_t)also_stride, post);
+  } else if (hidden % 4 == 0 && threads <= 1024) {
+    hipLaunchKernelGGL((add_rmsnorm_vec4_kernel<T, P, false>), dim3(out_rows), dim3(threads), 0, stream, (T*)y, residual,
+                       (const P*)pending, splits, (size_t)split_stride, (const T*)w, rows, eps, hidden, gain_offset,
+                       one_rounding, also, also_splits, (size_t)also_stride, post);
   } else {
     hipLaunchKernelGGL((add_rmsnorm_kernel<T, P>), dim3(out_rows), dim3(hidden <= 1024 ? 256 : 1024), 0, stream,
                        (T*)y, residual, (const P*)pending, splits, (size_t)split_stride, (const T*)w, rows, eps,
-                       hidden, gain_offset, one_rounding, also, also_splits, (size_t)also_stride);
+                       hidden, gain_offset, one_rounding, also, also_splits, (size_t)also_stride, post);
   }
 }
 
 // `out_rows` = rows of y written: the number of entries of `rows` if given, else the tokens.
 // pending_f32 != 0: `pending` holds `splits` 32-bit partial sums, `split_stride` elements apart.
 // `also`: a second addend, `also_splits` 32-bit partial sums `also_stride` apart (a block whose two parts
-// both add to the stream), or null.
+// both add to the stream), or null.  `post_gain` [hidden] of the run type, or null: the pending output is
+// divided by its root mean square (`post_eps` inside the root) and multiplied by the gain and by
+// `post_scale` before it is added.
 extern "C" int ts_add_rmsnorm(void* y, float* residual, const void* pending, int pending_f32, int splits,
                               long split_stride, const void* w, const int* rows, float eps, int out_rows,
                               int hidden, float gain_offset, int one_rounding, int dtype, const float* also,
-                              int also_splits, long also_stride, hipStream_t stream) {
+                              int also_splits, long also_stride, const void* post_gain, float post_eps,
+                              float post_scale, hipStream_t stream) {
   if (out_rows == 0) return TS_OK;
   if (!y || !residual || !w || hidden < 1 || splits < 1 || (also && also_splits < 1)) return TS_ERR_ARG;
+  if (post_gain && (!pending || also)) return TS_ERR_ARG;
   if (dtype == TS_F32)
-    launch_add_rmsnorm<float, float>(y, residual, pending, splits, split_stride, w, rows, eps, out_rows, hidden, gain_offset, one_rounding, also, also_splits, also_stride, stream);
+    launch_add_rmsnorm<float, float>(y, residual, pending, splits, split_stride, w, rows, eps, out_rows, hidden, gain_offset, one_rounding, also, also_splits, also_stride, post_gain, post_eps, post_scale, stream);
   else if (dtype == TS_BF16 && pending_f32)
-    launch_add_rmsnorm<bf16_t, float>(y, residual, pending, splits, split_stride, w, rows, eps, out_rows, hidden, gain_offset, one_rounding, also, also_splits, also_stride, stream);
+    launch_add_rmsnorm<bf16_t, float>(y, residual, pending, splits, split_stride, w, rows, eps, out_rows, hidden, gain_offset, one_rounding, also, also_splits, also_stride, post_gain, post_eps, post_scale, stream);
   else if (dtype == TS_BF16)
-    launch_add_rmsnorm<bf16_t, bf16_t>(y, residual, pending, splits, split_stride, w, rows, eps, out_rows, hidden, gain_offset, one_rounding, also, also_splits, also_stride, stream);
+    launch_add_rmsnorm<bf16_t, bf16_t>(y, residual, pending, splits, split_stride, w, rows, eps, out_rows, hidden, gain_offset, one_rounding, also, also_splits, also_stride, post_gain, post_eps, post_scale, stream);
   else
     return TS_ERR_DTYPE;
   return ts_launch_status();
@@ -717,5 +796,72 @@ extern "C" int ts_copy_f32(float* out, const float* in, long total, hipStream_t 
   if (total == 0) return TS_OK;
   if (!out || !in || total < 0) return TS_ERR_ARG;
   hipLaunchKernelGGL(copy_f32_kernel, dim3((unsigned)((total + 255) / 256)), dim3(256), 0, stream, out, in, (size_t)total);
+  return ts_launch_status();
+}
+
+// ---------------------------------------------------------------------------------------------
+// An activation over a projection output [T, I] (of type T, or `splits` 32-bit partial sums that are
+// added up here): out[t, i] = act(x[t, i]), computed in 32-bit and rounded once.  For feed-forwards
+// without a gate: down(act(up(x))).
+//   kind 0: relu(x)^2     kind 1: relu(x)     kind 2: x sigmoid(x)
+//   kind 3: the tanh form of GELU, 0.5 x (1 + tanh(sqrt(2 / pi) (x + 0.044715 x^3)))
+// ---------------------------------------------------------------------------------------------
+__device__ __forceinline__ float activation(float x, int kind) {
+  if (kind == 0) {
+    const float r = fmaxf(x, 0.f);
+    return r * r;
+  }
+  if (kind == 1) return fmaxf(x, 0.f);
+  if (kind == 2) return x / (1.f + expf(-x));
+  return x / (1.f + expf(-1.5957691216057308f * fmaf(0.044715f * x * x, x, x)));
+}
+
+template <typename T, typename P>
+__global__ void activate_kernel(T* __restrict__ out, const P* __restrict__ x, int splits, size_t split_stride,
+                                size_t total, int kind) {
+  const size_t idx = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
+  if (idx >= total) return;
+  out[idx] = from_float<T>(activation(add_splits(x + idx, splits, split_stride, 0.f), kind));
+}
+
+template <typename T, typename P>
+__global__ void activate_vec4_kernel(T* __restrict__ out, const P* __restrict__ x, int splits, size_t split_stride,
+                                     size_t quads, int kind) {
+  const size_t idx = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
+  if (idx >= quads) return;
+  float s[4] = {0.f, 0.f, 0.f, 0.f};
+  add_splits4(x + 4 * idx, splits, split_stride, s);
+  float o[4];
+#pragma unroll
+  for (int e = 0; e < 4; ++e) o[e] = activation(s[e], kind);
+  Vec4Of<T>::store(out + 4 * idx, o);
+}
+
+template <typename T, typename P>
+static void launch_activate(void* out, const void* x, int splits, long split_stride, size_t total, int kind,
+                            hipStream_t stream) {
+  if (total % 4 == 0 && ((uintptr_t)out | (uintptr_t)x) % 16 == 0 && split_stride % 4 == 0) {
+    const size_t quads = total / 4;
+    hipLaunchKernelGGL((activate_vec4_kernel<T, P>), dim3((unsigned)((quads + 255) / 256)), dim3(256), 0, stream, (T*)out,
+                       (const P*)x, splits, (size_t)split_stride, quads, kind);
+  } else {
+    hipLaunchKernelGGL((activate_kernel<T, P>), dim3((unsigned)((total + 255) / 256)), dim3(256), 0, stream, (T*)out,
+                       (const P*)x, splits, (size_t)split_stride, total, kind);
+  }
+}
+
+extern "C" int ts_activate(void* out, const void* x, int in_f32, int splits, long split_stride, int tokens, int inter,
+                           int kind, int dtype, hipStream_t stream) {
+  if (tokens == 0) return TS_OK;
+  if (!out || !x || inter < 1 || splits < 1 || kind < 0 || kind > 3) return TS_ERR_ARG;
+  const size_t total = (size_t)tokens * inter;
+  if (dtype == TS_F32)
+    launch_activate<float, float>(out, x, splits, split_stride, total, kind, stream);
+  else if (dtype == TS_BF16 && in_f32)
+    launch_activate<bf16_t, float>(out, x, splits, split_stride, total, kind, stream);
+  else if (dtype == TS_BF16)
+    launch_activate<bf16_t, bf16_t>(out, x, 1, 0, total, kind, stream);
+  else
+    return TS_ERR_DTYPE;
   return ts_launch_status();
 }

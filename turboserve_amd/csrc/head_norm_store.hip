@@ -10,12 +10,27 @@
 // projection of type T this may be the projection itself), keys to key pages [NB, Hkv, BS, D] at
 // slot = page * BS + offset, values to the transposed value pages [NB, Hkv, Dv, BS].  A negative
 // slot or slots == nullptr: nothing is stored for that token.
+//
+// Values may be blended with another layer's values of the same tokens before they are stored
+// (ValueBlend): `keep` [T, Hkv Dv] 32-bit, if given, receives this layer's values as projected;
+// `other` [T, Hkv Dv] 32-bit, if given, makes the stored value (1 - weight) v + weight other, in 32-bit.
 #include <type_traits>
 
 #include "common.hpp"
 
 #define HNS_MAX_DIM 512
 #define HNS_WAVES 4
+
+struct ValueBlend {
+  float* keep;
+  const float* other;
+  float weight;
+};
+
+__device__ __forceinline__ float blended(float v, size_t at, ValueBlend blend) {
+  if (blend.keep) blend.keep[at] = v;
+  return blend.other ? fmaf(blend.weight, blend.other[at], (1.f - blend.weight) * v) : v;
+}
 
 template <typename P>
 __device__ __forceinline__ float sum_of_splits(const P* p, int splits, size_t stride) {
@@ -42,7 +57,7 @@ head_norm_store_kernel(T* q_out, long q_stride, const P* proj, int splits, size_
                        float eps, float gain_offset, const float* __restrict__ cos_table,
                        const float* __restrict__ sin_table, const int* __restrict__ positions,
                        const int* __restrict__ slots, int tokens, int heads, int kv_heads, int dim, int vdim,
-                       int block_size) {
+                       int block_size, ValueBlend blend) {
   __shared__ float held[HNS_WAVES][HNS_MAX_DIM];
   const int wave = threadIdx.x / TS_WAVE, lane = threadIdx.x % TS_WAVE;
   const int qk_heads = heads + kv_heads;
@@ -58,8 +73,9 @@ head_norm_store_kernel(T* q_out, long q_stride, const P* proj, int splits, size_
       const int kvh = item_head - qk_heads;
       const P* values = proj + (size_t)item_token * width + (size_t)qk_heads * dim + (size_t)kvh * vdim;
       T* page = v_pages + ((size_t)(slot / block_size) * kv_heads + kvh) * vdim * block_size + slot % block_size;
+      const size_t at = ((size_t)item_token * kv_heads + kvh) * vdim;
       for (int d = lane; d < vdim; d += TS_WAVE)
-        page[(size_t)d * block_size] = from_float<T>(sum_of_splits(values + d, splits, split_stride));
+        page[(size_t)d * block_size] = from_float<T>(blended(sum_of_splits(values + d, splits, split_stride), at + d, blend));
     }
   }
   // (A value wavefront goes on as an idle one: the barrier below is the whole block's.)
@@ -194,7 +210,7 @@ template <typename T, typename P>
 __global__ void __launch_bounds__(64)
 value_store_kernel(const P* proj, int splits, size_t split_stride, T* __restrict__ v_pages,
                    const int* __restrict__ slots, int tokens, int heads, int kv_heads, int dim, int vdim,
-                   int block_size) {
+                   int block_size, ValueBlend blend) {
   const int t0 = blockIdx.x * HNS_GROUP;
   const int kvh = blockIdx.y;
   const int count = min(HNS_GROUP, tokens - t0);
@@ -210,7 +226,9 @@ value_store_kernel(const P* proj, int splits, size_t split_stride, T* __restrict
     alignas(16) T v[HNS_GROUP];
 #pragma unroll
     for (int j = 0; j < HNS_GROUP; ++j)
-      v[j] = from_float<T>(j < count ? sum_of_splits(column + (size_t)j * width + d, splits, split_stride) : 0.f);
+      v[j] = from_float<T>(j < count ? blended(sum_of_splits(column + (size_t)j * width + d, splits, split_stride),
+                                               ((size_t)(t0 + j) * kv_heads + kvh) * vdim + d, blend)
+                                     : 0.f);
     if (run) {
       T* dst = v_pages + (((size_t)(slot[0] / block_size) * kv_heads + kvh) * vdim + d) * block_size + slot[0] % block_size;
       *reinterpret_cast<uint4*>(dst) = *reinterpret_cast<const uint4*>(v);
@@ -229,7 +247,7 @@ static void launch_head_norm_store(void* q_out, long q_stride, const void* proj,
                                    void* k_pages, void* v_pages, const void* q_gain, const void* k_gain, float eps,
                                    float gain_offset, const float* cos_table, const float* sin_table,
                                    const int* positions, const int* slots, int tokens, int heads, int kv_heads,
-                                   int dim, int vdim, int block_size, hipStream_t stream) {
+                                   int dim, int vdim, int block_size, ValueBlend blend, hipStream_t stream) {
   const bool few = tokens < 4 * HNS_GROUP || splits > 1;  // values in the same launch, a wavefront per value head
   const long items = (long)tokens * (heads + kv_heads + (few && slots ? kv_heads : 0));
   const bool aligned = ((uintptr_t)q_out | (uintptr_t)proj | (uintptr_t)k_pages | (uintptr_t)q_gain | (uintptr_t)k_gain) % 16 == 0 &&
@@ -243,11 +261,11 @@ static void launch_head_norm_store(void* q_out, long q_stride, const void* proj,
     hipLaunchKernelGGL((head_norm_store_kernel<T, P>), dim3((unsigned)((items + HNS_WAVES - 1) / HNS_WAVES)),
                        dim3(64 * HNS_WAVES), 0, stream, (T*)q_out, q_stride, (const P*)proj, splits, (size_t)split_stride,
                        (T*)k_pages, (T*)v_pages, few && slots ? 1 : 0, (const T*)q_gain, (const T*)k_gain, eps, gain_offset,
-                       cos_table, sin_table, positions, slots, tokens, heads, kv_heads, dim, vdim, block_size);
+                       cos_table, sin_table, positions, slots, tokens, heads, kv_heads, dim, vdim, block_size, blend);
   if (slots && !few)
     hipLaunchKernelGGL((value_store_kernel<T, P>), dim3((tokens + HNS_GROUP - 1) / HNS_GROUP, kv_heads), dim3(64), 0,
                        stream, (const P*)proj, splits, (size_t)split_stride, (T*)v_pages, slots, tokens, heads, kv_heads,
-                       dim, vdim, block_size);
+                       dim, vdim, block_size, blend);
 }
 
 extern "C" int ts_head_norm_store(void* q_out, long q_stride, const void* proj, int in_f32, int splits,
@@ -255,8 +273,10 @@ extern "C" int ts_head_norm_store(void* q_out, long q_stride, const void* proj, 
                                   const void* k_gain, float eps, float gain_offset, const float* cos_table,
                                   const float* sin_table, const int* positions, const int* slots, int tokens,
                                   int heads, int kv_heads, int dim, int vdim, int block_size, int dtype,
-                                  hipStream_t stream) {
+                                  float* v_keep, const float* v_other, float v_weight, hipStream_t stream) {
   if (tokens == 0) return TS_OK;
+  if ((v_keep || v_other) && !slots) return TS_ERR_ARG;  // values are only walked where they are stored
+  const ValueBlend blend = {v_keep, v_other, v_weight};
   if (!q_out || !proj || !positions || heads < 1 || kv_heads < 1 || dim < 1 || dim > HNS_MAX_DIM || vdim < 1 ||
       block_size < 1 || splits < 1 || kv_heads > 65535)
     return TS_ERR_ARG;
@@ -264,11 +284,11 @@ extern "C" int ts_head_norm_store(void* q_out, long q_stride, const void* proj, 
   if ((q_gain == nullptr) != (k_gain == nullptr)) return TS_ERR_ARG;
   if (slots && (!k_pages || !v_pages)) return TS_ERR_ARG;
   if (dtype == TS_F32)
-    launch_head_norm_store<float, float>(q_out, q_stride, proj, splits, split_stride, k_pages, v_pages, q_gain, k_gain, eps, gain_offset, cos_table, sin_table, positions, slots, tokens, heads, kv_heads, dim, vdim, block_size, stream);
+    launch_head_norm_store<float, float>(q_out, q_stride, proj, splits, split_stride, k_pages, v_pages, q_gain, k_gain, eps, gain_offset, cos_table, sin_table, positions, slots, tokens, heads, kv_heads, dim, vdim, block_size, blend, stream);
   else if (dtype == TS_BF16 && in_f32)
-    launch_head_norm_store<bf16_t, float>(q_out, q_stride, proj, splits, split_stride, k_pages, v_pages, q_gain, k_gain, eps, gain_offset, cos_table, sin_table, positions, slots, tokens, heads, kv_heads, dim, vdim, block_size, stream);
+    launch_head_norm_store<bf16_t, float>(q_out, q_stride, proj, splits, split_stride, k_pages, v_pages, q_gain, k_gain, eps, gain_offset, cos_table, sin_table, positions, slots, tokens, heads, kv_heads, dim, vdim, block_size, blend, stream);
   else if (dtype == TS_BF16)
-    launch_head_norm_store<bf16_t, bf16_t>(q_out, q_stride, proj, splits, split_stride, k_pages, v_pages, q_gain, k_gain, eps, gain_offset, cos_table, sin_table, positions, slots, tokens, heads, kv_heads, dim, vdim, block_size, stream);
+    launch_head_norm_store<bf16_t, bf16_t>(q_out, q_stride, proj, splits, split_stride, k_pages, v_pages, q_gain, k_gain, eps, gain_offset, cos_table, sin_table, positions, slots, tokens, heads, kv_heads, dim, vdim, block_size, blend, stream);
   else
     return TS_ERR_DTYPE;
   return ts_launch_status();

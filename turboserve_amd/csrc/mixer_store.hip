@@ -6,6 +6,7 @@
 //                        vector is normalised, the shared rotated key part and the queries' rotated
 //                        parts are turned by the position's angles, latent and rotated key go into
 //                        the key pages as one row, the queries are split for what follows;
+//   ts_head_gate         every head's output times the sigmoid of a gate column of the projection;
 //   ts_stream_fold       residual (+)= a part's output (a tensor of the run type or 32-bit partial sums);
 //   ts_stream_pair       [x | origin] of two 32-bit streams side by side, in the run type.
 //
@@ -112,9 +113,10 @@ extern "C" int ts_span_norm_store(void* q_out, long q_stride, const void* proj, 
 
 // ---------------------------------------------------------------------------------------------
 // One block per token.  Row of the projection: [H (D plain | R rotated) queries | C latent | R
-// rotated key].  Of a rotated part the first `turned` elements are turned in pairs (i, i +
-// turned / 2) by the angles of the token's position (tables [capacity, turned / 2], 32-bit); the
-// rest pass unchanged.
+// rotated key | `tail` more columns that are not read here].  Of a rotated part the first `turned`
+// elements are turned in pairs (i, i + turned / 2), or with `neighbours` in pairs (2 i, 2 i + 1), by
+// the angles of the token's position (tables [capacity, turned / 2], 32-bit, which may carry a
+// factor on both the cosine and the sine); the rest pass unchanged.
 //   key page row [NB, 1, BS, C + R] at the token's slot  <- [latent * rsqrt(mean(latent^2) + eps) * gain | turned key]
 //   q_plain [T H, D]                                     <- the queries' plain parts
 //   q_wide  [T, H, C + R], elements C..C+R-1 only        <- the queries' turned parts
@@ -122,9 +124,14 @@ extern "C" int ts_span_norm_store(void* q_out, long q_stride, const void* proj, 
 // product writes afterwards).
 // ---------------------------------------------------------------------------------------------
 __device__ __forceinline__ float turned_element(const float* part, int i, int turned, const float* cos_row,
-                                                const float* sin_row) {
+                                                const float* sin_row, int neighbours) {
   const int half = turned / 2;
   if (i >= turned) return part[i];
+  if (neighbours) {  // pairs (2 j, 2 j + 1), angle j
+    const int j = i / 2;
+    if ((i & 1) == 0) return __builtin_fmaf(part[i], cos_row[j], -(part[i + 1] * sin_row[j]));
+    return __builtin_fmaf(part[i], cos_row[j], part[i - 1] * sin_row[j]);
+  }
   if (i < half) return __builtin_fmaf(part[i], cos_row[i], -(part[i + half] * sin_row[i]));
   return __builtin_fmaf(part[i], cos_row[i - half], part[i - half] * sin_row[i - half]);
 }
@@ -135,13 +142,13 @@ latent_store_kernel(T* __restrict__ q_plain, T* __restrict__ q_wide, const P* pr
                     T* __restrict__ k_pages, const T* __restrict__ gain, float eps,
                     const float* __restrict__ cos_table, const float* __restrict__ sin_table,
                     const int* __restrict__ positions, const int* __restrict__ slots, int heads, int dim,
-                    int rot, int rank, int turned, int block_size) {
+                    int rot, int rank, int turned, int block_size, int neighbours, int tail) {
   extern __shared__ float held[];  // [heads * rot] the queries' rotated parts, [rot] the key's, then the latent
   __shared__ float scratch[16];
   const int t = blockIdx.x;
   const int per_head = dim + rot;
   const int q_size = heads * per_head;
-  const P* row = proj + (size_t)t * (q_size + rank + rot);
+  const P* row = proj + (size_t)t * (q_size + rank + rot + tail);
   float* q_rot = held;
   float* k_rot = held + heads * rot;
   float* latent = k_rot + rot;
@@ -166,45 +173,80 @@ latent_store_kernel(T* __restrict__ q_plain, T* __restrict__ q_wide, const P* pr
   }
   for (int i = threadIdx.x; i < heads * rot; i += blockDim.x) {
     const int h = i / rot, d = i % rot;
-    q_wide[((size_t)t * heads + h) * wide + rank + d] = from_float<T>(turned_element(q_rot + h * rot, d, turned, cos_row, sin_row));
+    q_wide[((size_t)t * heads + h) * wide + rank + d] = from_float<T>(turned_element(q_rot + h * rot, d, turned, cos_row, sin_row, neighbours));
   }
   const int slot = slots ? slots[t] : -1;
   if (slot < 0) return;
   T* dst = k_pages + (size_t)slot * wide;  // one key head: row `slot` of [NB * BS, C + R]
   for (int i = threadIdx.x; i < rank; i += blockDim.x) dst[i] = from_float<T>(latent[i] * r * to_float(gain[i]));
   for (int i = threadIdx.x; i < rot; i += blockDim.x)
-    dst[rank + i] = from_float<T>(turned_element(k_rot, i, turned, cos_row, sin_row));
+    dst[rank + i] = from_float<T>(turned_element(k_rot, i, turned, cos_row, sin_row, neighbours));
 }
 
 template <typename T, typename P>
 static int latent_store_launch(void* q_plain, void* q_wide, const void* proj, int splits, long split_stride, void* k_pages,
                                const void* gain, float eps, const float* cos_table, const float* sin_table,
                                const int* positions, const int* slots, int tokens, int heads, int dim, int rot, int rank,
-                               int turned, int block_size, hipStream_t stream) {
+                               int turned, int block_size, int neighbours, int tail, hipStream_t stream) {
   const size_t lds = (size_t)(heads * rot + rot + rank) * sizeof(float);
   if (lds > 60 * 1024) return TS_ERR_SHAPE;
   hipLaunchKernelGGL((latent_store_kernel<T, P>), dim3(tokens), dim3(tokens <= 64 ? 1024 : 256), lds, stream, (T*)q_plain, (T*)q_wide,
                      (const P*)proj, splits, (size_t)split_stride, (T*)k_pages, (const T*)gain, eps, cos_table, sin_table,
-                     positions, slots, heads, dim, rot, rank, turned, block_size);
+                     positions, slots, heads, dim, rot, rank, turned, block_size, neighbours, tail);
   return ts_launch_status();
 }
 
 extern "C" int ts_latent_store(void* q_plain, void* q_wide, const void* proj, int in_f32, int splits, long split_stride,
                                void* k_pages, const void* gain, float eps, const float* cos_table,
                                const float* sin_table, const int* positions, const int* slots, int tokens, int heads,
-                               int dim, int rot, int rank, int turned, int block_size, int dtype, hipStream_t stream) {
+                               int dim, int rot, int rank, int turned, int block_size, int neighbours, int tail, int dtype,
+                               hipStream_t stream) {
   if (tokens == 0) return TS_OK;
   if (!q_plain || !q_wide || !proj || !gain || !cos_table || !sin_table || !positions || (slots && !k_pages))
     return TS_ERR_ARG;
-  if (heads < 1 || dim < 1 || rot < 1 || rank < 1 || turned < 2 || turned > rot || (turned & 1) || block_size < 1 || splits < 1)
+  if (heads < 1 || dim < 1 || rot < 1 || rank < 1 || turned < 2 || turned > rot || (turned & 1) || block_size < 1 || splits < 1 || tail < 0)
     return TS_ERR_SHAPE;
   if (dtype == TS_F32)
-    return latent_store_launch<float, float>(q_plain, q_wide, proj, splits, split_stride, k_pages, gain, eps, cos_table, sin_table, positions, slots, tokens, heads, dim, rot, rank, turned, block_size, stream);
+    return latent_store_launch<float, float>(q_plain, q_wide, proj, splits, split_stride, k_pages, gain, eps, cos_table, sin_table, positions, slots, tokens, heads, dim, rot, rank, turned, block_size, neighbours, tail, stream);
   if (dtype == TS_BF16 && in_f32)
-    return latent_store_launch<bf16_t, float>(q_plain, q_wide, proj, splits, split_stride, k_pages, gain, eps, cos_table, sin_table, positions, slots, tokens, heads, dim, rot, rank, turned, block_size, stream);
+    return latent_store_launch<bf16_t, float>(q_plain, q_wide, proj, splits, split_stride, k_pages, gain, eps, cos_table, sin_table, positions, slots, tokens, heads, dim, rot, rank, turned, block_size, neighbours, tail, stream);
   if (dtype == TS_BF16)
-    return latent_store_launch<bf16_t, bf16_t>(q_plain, q_wide, proj, 1, 0, k_pages, gain, eps, cos_table, sin_table, positions, slots, tokens, heads, dim, rot, rank, turned, block_size, stream);
+    return latent_store_launch<bf16_t, bf16_t>(q_plain, q_wide, proj, 1, 0, k_pages, gain, eps, cos_table, sin_table, positions, slots, tokens, heads, dim, rot, rank, turned, block_size, neighbours, tail, stream);
   return TS_ERR_DTYPE;
+}
+
+// ---------------------------------------------------------------------------------------------
+// out [T, H, Dv] of the run type: head h's row of the 32-bit `values` [T, H, Dv] times the sigmoid of
+// the head's gate, which is column gate_at + h of the token's row of a projection (`width` columns; of
+// type T, or `splits` 32-bit partial sums).  32-bit arithmetic, one rounding.
+// ---------------------------------------------------------------------------------------------
+template <typename T, typename P>
+__global__ void __launch_bounds__(256)
+head_gate_kernel(T* __restrict__ out, const float* __restrict__ values, const P* __restrict__ proj, int splits,
+                 size_t split_stride, int width, int gate_at, int heads, int vdim) {
+  const int t = blockIdx.x;
+  const int per = heads * vdim;
+  for (int i = threadIdx.x; i < per; i += blockDim.x) {
+    const float g = folded(proj + (size_t)t * width + gate_at + i / vdim, splits, split_stride);
+    out[(size_t)t * per + i] = from_float<T>(values[(size_t)t * per + i] / (1.f + expf(-g)));
+  }
+}
+
+extern "C" int ts_head_gate(void* out, const float* values, const void* proj, int in_f32, int splits, long split_stride,
+                            int tokens, int width, int gate_at, int heads, int vdim, int dtype, hipStream_t stream) {
+  if (tokens == 0) return TS_OK;
+  if (!out || !values || !proj || heads < 1 || vdim < 1 || splits < 1 || gate_at < 0 || gate_at + heads > width)
+    return TS_ERR_ARG;
+  const dim3 grid(tokens), block(256);
+  if (dtype == TS_F32)
+    hipLaunchKernelGGL((head_gate_kernel<float, float>), grid, block, 0, stream, (float*)out, values, (const float*)proj, splits, (size_t)split_stride, width, gate_at, heads, vdim);
+  else if (dtype == TS_BF16 && in_f32)
+    hipLaunchKernelGGL((head_gate_kernel<bf16_t, float>), grid, block, 0, stream, (bf16_t*)out, values, (const float*)proj, splits, (size_t)split_stride, width, gate_at, heads, vdim);
+  else if (dtype == TS_BF16)
+    hipLaunchKernelGGL((head_gate_kernel<bf16_t, bf16_t>), grid, block, 0, stream, (bf16_t*)out, values, (const bf16_t*)proj, 1, (size_t)0, width, gate_at, heads, vdim);
+  else
+    return TS_ERR_DTYPE;
+  return ts_launch_status();
 }
 
 // ---------------------------------------------------------------------------------------------

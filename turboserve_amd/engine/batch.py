@@ -343,6 +343,10 @@ class StepContext:
     recorded: bool = False
     #: The fields the model's parts asked for (``Part.step_fields``), by name: int32 device views.
     extras: dict = field(default_factory=dict)
+    #: Device tensors one layer makes in this step for a later layer of the same step (by a key the
+    #: two agree on): values an earlier layer projected that a later one mixes into its own.  They
+    #: are the step's own intermediates, so a recorded step holds them like any other.
+    carried: dict = field(default_factory=dict, repr=False)
     _derived: dict = field(default_factory=dict, repr=False)
 
     def derive(self, key: Hashable, make: Callable[["StepContext"], Any]) -> Any:

@@ -60,28 +60,32 @@ _SIGNATURES: dict[str, dict[str, list]] = {
         "ts_embed": [c_void_p, c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_void_p],
         "ts_rmsnorm": [c_void_p, c_void_p, c_void_p, c_float, c_int, c_int, c_float, c_int, c_int, c_void_p],
         "ts_add_rmsnorm": [c_void_p, c_void_p, c_void_p, c_int, c_int, c_long, c_void_p, c_void_p, c_float,
-                           c_int, c_int, c_float, c_int, c_int, c_void_p, c_int, c_long, c_void_p],
+                           c_int, c_int, c_float, c_int, c_int, c_void_p, c_int, c_long, c_void_p, c_float, c_float, c_void_p],
         "ts_swiglu": [c_void_p, c_void_p, c_int, c_int, c_long, c_int, c_int, c_int, c_float, c_float, c_float, c_float, c_int,
                       c_void_p],
+        "ts_activate": [c_void_p, c_void_p, c_int, c_int, c_long, c_int, c_int, c_int, c_int, c_void_p],
         "ts_rope_store": [c_void_p, c_long, c_void_p, c_int, c_int, c_long, c_void_p, c_void_p, c_void_p, c_void_p,
                           c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_int, c_int, c_int, c_void_p],
         "ts_gather_rows": [c_void_p, c_void_p, c_void_p, c_int, c_int, c_int, c_void_p],
         "ts_patch_tokens": [c_void_p, c_void_p, c_void_p, c_int, c_int, c_void_p],
         "ts_paged_attention_generic": [c_void_p, c_void_p, c_long, c_void_p, c_void_p, c_void_p, c_int,
                                        c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_int, c_int,
-                                       c_float, c_float, c_int, c_void_p, c_int, c_float, c_int, c_void_p],
+                                       c_float, c_float, c_int, c_void_p, c_int, c_float, c_void_p, c_void_p, c_int, c_int,
+                                       c_void_p],
         "ts_attention_tiles": [c_void_p, c_void_p, c_void_p, c_void_p, c_long, c_void_p, c_void_p, c_void_p, c_int, c_void_p,
                                c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_int, c_int, c_int, c_float, c_float, c_int,
-                               c_int, c_float, c_void_p, c_int, c_int, c_void_p],
+                               c_int, c_float, c_void_p, c_int, c_int, c_void_p, c_void_p, c_int, c_void_p],
         "ts_attention_tiles_combine": [c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_int, c_float,
-                                       c_void_p],
+                                       c_void_p, c_void_p],
         "ts_head_norm_store": [c_void_p, c_long, c_void_p, c_int, c_int, c_long, c_void_p, c_void_p, c_void_p, c_void_p,
                                c_float, c_float, c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_int, c_int, c_int,
-                               c_int, c_int, c_int, c_void_p],
+                               c_int, c_int, c_int, c_void_p, c_void_p, c_float, c_void_p],
         "ts_span_norm_store": [c_void_p, c_long, c_void_p, c_int, c_int, c_long, c_void_p, c_void_p, c_void_p, c_void_p,
                                c_float, c_float, c_void_p, c_int, c_int, c_int, c_int, c_int, c_int, c_int, c_void_p],
         "ts_latent_store": [c_void_p, c_void_p, c_void_p, c_int, c_int, c_long, c_void_p, c_void_p, c_float, c_void_p,
-                            c_void_p, c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_int, c_int, c_int, c_int, c_void_p],
+                            c_void_p, c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_int, c_int, c_int, c_int, c_int, c_int,
+                            c_void_p],
+        "ts_head_gate": [c_void_p, c_void_p, c_void_p, c_int, c_int, c_long, c_int, c_int, c_int, c_int, c_int, c_int, c_void_p],
         "ts_stream_fold": [c_void_p, c_void_p, c_int, c_int, c_long, c_long, c_int, c_int, c_void_p],
         "ts_stream_pair": [c_void_p, c_void_p, c_void_p, c_int, c_int, c_int, c_void_p],
         "ts_linear_state_scan": [c_void_p, c_void_p, c_int, c_int, c_long, c_void_p, c_void_p, c_float, c_void_p, c_void_p,
@@ -421,11 +425,15 @@ class Ops:
         gain_offset: float = 0.0,
         one_rounding: bool = False,
         also: torch.Tensor | None = None,
+        pending_norm: tuple[torch.Tensor, float, float] | None = None,
     ) -> torch.Tensor:
         """``residual += pending`` in 32-bit (in place) and the normalised sum in ``weight``'s
         dtype; with ``rows`` only those rows, and ``residual`` is left alone.  ``pending`` is a
         ``[T, H]`` tensor of the run dtype or ``[S, T, H]`` 32-bit partial sums.  ``also``: a second
-        addend, ``[S, T, H]`` 32-bit partial sums.  The gain is applied as in :meth:`rmsnorm`."""
+        addend, ``[S, T, H]`` 32-bit partial sums.  The gain is applied as in :meth:`rmsnorm`.
+        ``pending_norm = (gain [H], eps, scale)``: the pending output is first divided by its own
+        root mean square (``eps`` inside the root) and multiplied by ``gain`` and ``scale``, in
+        32-bit, so what is added is ``scale * norm(pending)``."""
         _gpu(residual, pending, weight, rows)
         _i32(rows, "rows")
         _need(residual.dim() == 2 and residual.dtype == torch.float32 and residual.is_contiguous(),
@@ -441,12 +449,19 @@ class Ops:
             _need(also.dim() == 3 and also.dtype == torch.float32 and also.is_contiguous() and also.shape[1:] == (tokens, hidden),
                   "a second addend must be float32 partial sums [S, T, H]")
             also_splits, also_stride = also.shape[0], tokens * hidden
+        post_gain, post_eps, post_scale = None, 0.0, 1.0
+        if pending_norm is not None:
+            post_gain, post_eps, post_scale = pending_norm
+            _gpu(post_gain)
+            _need(pending is not None and also is None, "a norm on the pending output needs one, and no second addend")
+            _need(post_gain.shape == (hidden,) and post_gain.dtype == weight.dtype and post_gain.is_contiguous(),
+                  "the pending output's gain must be [H] of the run dtype")
         out_rows = tokens if rows is None else rows.numel()
         y = self.rows_buffer(out_rows, hidden, weight.dtype, residual.device)
         _check(self.core.ts_add_rmsnorm(_ptr(y), _ptr(residual), _ptr(pending), is_f32, splits, stride, _ptr(weight),
                                         _ptr(rows), float(eps), out_rows, hidden, float(gain_offset),
                                         1 if one_rounding else 0, dtype_code(weight.dtype), _ptr(also), also_splits,
-                                        also_stride, self.stream()),
+                                        also_stride, _ptr(post_gain), float(post_eps), float(post_scale), self.stream()),
                "ts_add_rmsnorm")
         return y
 
@@ -470,6 +485,25 @@ class Ops:
         _check(self.core.ts_swiglu(_ptr(out), _ptr(gate_up), is_f32, splits, stride, tokens, inter,
                                    1 if paired else 0, *glu_rule(rule),
                                    dtype_code(out_dtype), self.stream()), "ts_swiglu")
+        return out
+
+    #: The activations :meth:`activate` knows, by name.
+    ACTIVATIONS = {"relu_squared": 0, "relu": 1, "silu": 2, "gelu_tanh": 3}
+
+    def activate(self, proj: torch.Tensor, kind: str, dtype: torch.dtype | None = None) -> torch.Tensor:
+        """``act(proj)`` element by element, in 32-bit with one rounding: ``proj`` is a projection
+        ``[T, I]`` of the run dtype or its ``[S, T, I]`` 32-bit partial sums, the result ``[T, I]`` of
+        ``dtype``.  ``kind``: ``relu_squared`` (``max(x, 0)^2``), ``relu``, ``silu``, ``gelu_tanh``."""
+        _gpu(proj)
+        _need(kind in self.ACTIVATIONS, f"activation {kind!r} is not one of {sorted(self.ACTIVATIONS)}")
+        tokens, inter = proj.shape[-2], proj.shape[-1]
+        out_dtype = dtype or proj.dtype
+        if proj.dim() == 3:
+            _need(dtype is not None, "partial sums need the output dtype")
+        is_f32, splits, stride = self._partials(proj, tokens, inter, out_dtype, "projection")
+        out = self.rows_buffer(tokens, inter, out_dtype, proj.device)
+        _check(self.core.ts_activate(_ptr(out), _ptr(proj), is_f32, splits, stride, tokens, inter, self.ACTIVATIONS[kind],
+                                     dtype_code(out_dtype), self.stream()), "ts_activate")
         return out
 
     def gather_rows(self, x: torch.Tensor, rows: torch.Tensor) -> torch.Tensor:
@@ -612,14 +646,19 @@ class Ops:
         cos: torch.Tensor | None = None,
         sin: torch.Tensor | None = None,
         max_position: int = 0,
+        keep_values: torch.Tensor | None = None,
+        blend_values: tuple[torch.Tensor, float] | None = None,
     ) -> tuple[torch.Tensor, int]:
         """Per-head norm of the q and k heads of the fused projection ``[T, Hq D + Hkv D + Hkv Dv]``
         (``x * rsqrt(mean(x^2) + eps) * (gain_offset + gain)`` in 32-bit, the gain ``[D]`` shared by
         the heads; no norm without gains), then the rotation by ``cos``/``sin [capacity, D/2]`` where
         given, one rounding, and the store of k and v at ``slots`` into key pages ``[NB, Hkv, BS,
         D]`` and value pages ``[NB, Hkv, Dv, BS]`` (skipped when ``slots`` is ``None``).  Returns
-        the tensor that holds the queries and its row stride, as :meth:`rope_store` does."""
-        _gpu(proj, k_pages, v_pages, q_gain, k_gain, positions, slots, cos, sin)
+        the tensor that holds the queries and its row stride, as :meth:`rope_store` does.
+        ``keep_values [T, Hkv Dv]`` 32-bit receives the step's values as projected;
+        ``blend_values = (other [T, Hkv Dv] 32-bit, w)`` stores ``(1 - w) v + w other`` instead of ``v``
+        (another layer's values of the same tokens mixed in, in 32-bit)."""
+        _gpu(proj, k_pages, v_pages, q_gain, k_gain, positions, slots, cos, sin, keep_values)
         _i32(positions, "positions")
         _i32(slots, "slots")
         tokens = positions.numel()
@@ -650,10 +689,17 @@ class Ops:
             q_stride = heads * head_dim
         else:
             q_out, q_stride = proj, width
+        other, weight = (None, 0.0) if blend_values is None else blend_values
+        for held in (keep_values, other):
+            if held is not None:
+                _gpu(held)
+                _need(slots is not None and held.dtype == torch.float32 and held.is_contiguous()
+                      and held.shape == (tokens, kv_heads * value_dim), "values kept or mixed in are float32 [T, Hkv Dv], with slots")
         _check(self.core.ts_head_norm_store(
             _ptr(q_out), q_stride, _ptr(proj), is_f32, splits, stride, _ptr(k_pages), _ptr(v_pages), _ptr(q_gain),
             _ptr(k_gain), float(eps), float(gain_offset), _ptr(cos), _ptr(sin), _ptr(positions), _ptr(slots), tokens,
-            heads, kv_heads, head_dim, value_dim, block_size, dtype_code(run_dtype), self.stream()), "ts_head_norm_store")
+            heads, kv_heads, head_dim, value_dim, block_size, dtype_code(run_dtype), _ptr(keep_values), _ptr(other),
+            float(weight), self.stream()), "ts_head_norm_store")
         return q_out, q_stride
 
     # -- stores and stream steps of other mixers ------------------------------------------------
@@ -699,19 +745,21 @@ class Ops:
     def latent_store(self, proj: torch.Tensor, k_pages: torch.Tensor | None, gain: torch.Tensor, eps: float,
                      cos: torch.Tensor, sin: torch.Tensor, positions: torch.Tensor, slots: torch.Tensor | None,
                      heads: int, head_dim: int, rot_dim: int, rank: int, block_size: int, max_position: int,
-                     dtype: torch.dtype | None = None) -> tuple[torch.Tensor, torch.Tensor]:
+                     dtype: torch.dtype | None = None, *, neighbours: bool = False, tail: int = 0) -> tuple[torch.Tensor, torch.Tensor]:
         """A latent-attention layer's pass over its fused projection ``[T, H (D + R) + C + R]`` (per
         head ``D`` plain and ``R`` rotated query elements, then the latent of ``C`` and the shared
         rotated key part of ``R``): the latent is divided by its root mean square and multiplied by
         ``gain [C]``; of the rotated parts the first ``2 * cos.shape[1]`` elements are turned by the
         position's angles; ``[latent | rotated key]`` goes to the key pages ``[NB, 1, BS, C + R]`` at
         ``slots``.  Returns ``(q_plain [T H, D], q_wide [T, H, C + R])``; of ``q_wide`` only the last
-        ``R`` elements of every head are written (the turned query parts)."""
+        ``R`` elements of every head are written (the turned query parts).  ``neighbours``: the pairs
+        turned together are ``(2 i, 2 i + 1)`` instead of ``(i, i + turned / 2)``.  ``tail``: columns
+        behind the rotated key part in every row of the projection that this pass does not read."""
         _gpu(proj, k_pages, gain, cos, sin, positions, slots)
         _i32(positions, "positions")
         _i32(slots, "slots")
         tokens = positions.numel()
-        width = heads * (head_dim + rot_dim) + rank + rot_dim
+        width = heads * (head_dim + rot_dim) + rank + rot_dim + int(tail)
         run_dtype = dtype or proj.dtype
         if proj.dim() == 3:
             _need(dtype is not None, "partial sums need the run dtype")
@@ -730,8 +778,23 @@ class Ops:
         _check(self.core.ts_latent_store(
             _ptr(q_plain), _ptr(q_wide), _ptr(proj), is_f32, splits, stride, _ptr(k_pages), _ptr(gain), float(eps),
             _ptr(cos), _ptr(sin), _ptr(positions), _ptr(slots), tokens, heads, head_dim, rot_dim, rank, 2 * cos.shape[1],
-            block_size, dtype_code(run_dtype), self.stream()), "ts_latent_store")
+            block_size, 1 if neighbours else 0, int(tail), dtype_code(run_dtype), self.stream()), "ts_latent_store")
         return q_plain, q_wide
+
+    def head_gate(self, values: torch.Tensor, proj: torch.Tensor, gate_at: int, heads: int, dtype: torch.dtype) -> torch.Tensor:
+        """``[T, H Dv]`` of ``dtype``: head ``h``'s ``Dv`` elements of the 32-bit ``values [T, H Dv]`` times
+        ``sigmoid`` of column ``gate_at + h`` of the token's row of ``proj`` (a projection of the run
+        dtype or its 32-bit partial sums), in 32-bit with one rounding."""
+        _gpu(values, proj)
+        tokens, width = proj.shape[-2], proj.shape[-1]
+        is_f32, splits, stride = self._partials(proj, tokens, width, dtype, "projection")
+        _need(values.dtype == torch.float32 and values.is_contiguous() and values.dim() == 2 and values.shape[0] == tokens
+              and values.shape[1] % heads == 0 and 0 <= gate_at and gate_at + heads <= width,
+              "values must be float32 [T, H Dv] and the gates' columns inside the projection")
+        out = self.rows_buffer(tokens, values.shape[1], dtype, values.device)
+        _check(self.core.ts_head_gate(_ptr(out), _ptr(values), _ptr(proj), is_f32, splits, stride, tokens, width, gate_at,
+                                      heads, values.shape[1] // heads, dtype_code(dtype), self.stream()), "ts_head_gate")
+        return out
 
     def stream_fold(self, residual: torch.Tensor, part: torch.Tensor, dtype: torch.dtype, *, assign: bool = False) -> None:
         """``residual [T, H] += part`` in 32-bit, in place (``assign``: ``residual = part``); ``part`` is a
@@ -1037,6 +1100,8 @@ class Ops:
         chunk: int | None = None,
         sinks: float = 0.0,
         value_dim: int | None = None,
+        sink_scores: torch.Tensor | None = None,
+        distance_bias: torch.Tensor | None = None,
     ) -> torch.Tensor:
         """Attention of every token over the keys ``lo..position`` of its request.  With
         ``softcap = c > 0`` a scaled score ``s`` becomes ``c * tanh(s / c)``.  Values may have a
@@ -1047,8 +1112,11 @@ class Ops:
         score of key ``j`` for a query at position ``p`` by ``slopes[h] * (j - p)``.  ``chunk = C``:
         a query at ``p`` sees no key below ``(p // C) * C``.  ``sinks = n``: the softmax's denominator
         counts ``n`` more keys of score 0 that have no value.  ``v_pages = None`` with ``value_dim =
-        Dv <= D``: a key's value is its own first ``Dv`` elements."""
+        Dv <= D``: a key's value is its own first ``Dv`` elements.  ``sink_scores [heads]`` (32-bit):
+        the sinks' score per head instead of 0.  ``distance_bias [heads, L]`` (32-bit): the score of
+        the key ``n`` positions back gets ``distance_bias[h, min(n, L - 1)]`` added."""
         _gpu(q, k_pages, v_pages, block_table, token_seq, positions)
+        self._score_tables(heads, sinks, sink_scores, distance_bias)
         if slopes is not None:
             _gpu(slopes)
             _need(slopes.dtype == torch.float32 and slopes.is_contiguous() and slopes.numel() == heads,
@@ -1078,9 +1146,21 @@ class Ops:
             _ptr(out), _ptr(q), q_stride, _ptr(k_pages), _ptr(v_pages), _ptr(block_table),
             block_table.shape[1], _ptr(token_seq), _ptr(positions), tokens, heads, kv_heads, head_dim, value_dim,
             block_size, float(scale), float(softcap), int(window or 0), _ptr(slopes) if slopes is not None else None,
-            int(chunk or 0), float(sinks), dtype_code(q.dtype), self.stream()),
+            int(chunk or 0), float(sinks), _ptr(sink_scores), _ptr(distance_bias),
+            0 if distance_bias is None else distance_bias.shape[1], dtype_code(q.dtype), self.stream()),
             "ts_paged_attention_generic")
         return out
+
+    @staticmethod
+    def _score_tables(heads: int, sinks: float, sink_scores: torch.Tensor | None, distance_bias: torch.Tensor | None) -> None:
+        if sink_scores is not None:
+            _gpu(sink_scores)
+            _need(sinks > 0.0 and sink_scores.dtype == torch.float32 and sink_scores.is_contiguous()
+                  and sink_scores.shape == (heads,), "sink scores are float32 [heads] and go with a count of sinks")
+        if distance_bias is not None:
+            _gpu(distance_bias)
+            _need(distance_bias.dtype == torch.float32 and distance_bias.is_contiguous() and distance_bias.dim() == 2
+                  and distance_bias.shape[0] == heads and distance_bias.shape[1] >= 1, "a distance bias is float32 [heads, L]")
 
     @staticmethod
     def tiled_attention_supported(dtype: torch.dtype, head_dim: int, value_dim: int, block_size: int, q_stride: int,
@@ -1117,7 +1197,8 @@ class Ops:
                         tokens: int, heads: int, scale: float, prefill_tiles: torch.Tensor | None, num_prefill_seqs: int,
                         num_decode_seqs: int, max_decode_context: int, window: int | None = None, chunk: int | None = None,
                         sinks: float = 0.0, slopes: torch.Tensor | None = None, softcap: float = 0.0,
-                        value_dim: int | None = None) -> torch.Tensor:
+                        value_dim: int | None = None, sink_scores: torch.Tensor | None = None,
+                        distance_bias: torch.Tensor | None = None) -> torch.Tensor:
         """What :meth:`paged_attention_generic` computes, for bfloat16, on the matrix cores: the
         requests that bring several tokens (the first ``num_prefill_seqs``) in tiles of 64 tokens by
         one head (``prefill_tiles``: int32 ``[n, 2]`` from :meth:`attention_tile_list`), the
@@ -1125,6 +1206,8 @@ class Ops:
         their keys (at most ``max_decode_context``, a bound the step's shape gives) shared out over
         several workgroups.  Returns ``[T, heads * Dv]``."""
         _gpu(q, k_pages, v_pages, block_table, query_start_loc, context_lens, prefill_tiles, slopes)
+        self._score_tables(heads, sinks, sink_scores, distance_bias)
+        tables = (_ptr(sink_scores), _ptr(distance_bias), 0 if distance_bias is None else distance_bias.shape[1])
         _i32(block_table, "block_table")
         _i32(query_start_loc, "query_start_loc")
         _i32(context_lens, "context_lens")
@@ -1150,7 +1233,7 @@ class Ops:
         if num_prefill_seqs > 0:
             _need(prefill_tiles is not None and prefill_tiles.dim() == 2 and prefill_tiles.shape[1] == 2, "prefill_tiles [n, 2]")
             _check(self.core.ts_attention_tiles(_ptr(out), None, None, *common, _ptr(prefill_tiles), prefill_tiles.shape[0], 0,
-                                                heads, kv_heads, head_dim, value_dim, block_size, *rule, 0, 1, self.stream()),
+                                                heads, kv_heads, head_dim, value_dim, block_size, *rule, 0, 1, *tables, self.stream()),
                    "ts_attention_tiles")
         if num_decode_seqs > 0:
             # Workgroups per (request, KV head): enough to give every compute unit one, no more than the
@@ -1164,11 +1247,12 @@ class Ops:
                 partial_ml = torch.empty((num_decode_seqs, heads, splits, 2), dtype=torch.float32, device=q.device)
             _check(self.core.ts_attention_tiles(_ptr(out), _ptr(partial_o), _ptr(partial_ml), *common, None, num_decode_seqs,
                                                 num_prefill_seqs, heads, kv_heads, head_dim, value_dim, block_size, *rule, 1,
-                                                splits, self.stream()), "ts_attention_tiles")
+                                                splits, *tables, self.stream()), "ts_attention_tiles")
             if splits > 1:
                 _check(self.core.ts_attention_tiles_combine(_ptr(out), _ptr(partial_o), _ptr(partial_ml), _ptr(query_start_loc),
                                                             num_decode_seqs, num_prefill_seqs, heads, value_dim, splits,
-                                                            float(sinks), self.stream()), "ts_attention_tiles_combine")
+                                                            float(sinks), _ptr(sink_scores), self.stream()),
+                       "ts_attention_tiles_combine")
         return out
 
     @staticmethod

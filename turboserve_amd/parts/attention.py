@@ -48,7 +48,12 @@ class GroupedQueryAttention(Mixer):
     D]``, stored under the same names as the per-head gains); ``chunk = C`` (the token at position
     ``i`` sees only keys from ``(i // C) * C`` on: chunks of positions counted from the request's
     start); ``sinks = n`` (the softmax's denominator counts ``n`` more keys of score 0 that have no
-    value).  ``names``: the tensor
+    value); ``sink_name``: the sinks' score is learned, one number per query head in the tensor of
+    that name ``[Hq]`` (it is not scaled and gets no bias), instead of 0; ``value_mix = {"key": k,
+    "source": bool, "name": n}``: the layers of a model that share ``key`` mix their values: the one
+    marked ``source`` (the first of them to run) leaves its values as projected for the others of the
+    same step, and every other stores and attends over ``(1 - w) v + w v_source`` with its own learned
+    scalar ``w`` (tensor ``n``).  ``names``: the tensor
     names under the part's prefix of ``q, k, v, o`` (biases: the same with ``weight`` replaced by
     ``bias``) and of the two gains."""
 
@@ -73,6 +78,8 @@ class GroupedQueryAttention(Mixer):
         span_norm: Mapping | None = None,
         chunk: int | None = None,
         sinks: float = 0.0,
+        sink_name: str | None = None,
+        value_mix: Mapping | None = None,
     ) -> None:
         super().__init__(prefix, runtime)
         # Refused here, when the model is put together, not at the first step after the weights
@@ -105,6 +112,14 @@ class GroupedQueryAttention(Mixer):
         self.sinks = float(sinks)
         if self.sinks < 0:
             raise ValueError(f"{prefix or 'attention'}: {self.sinks} sinks")
+        self.sink_name = sink_name
+        if sink_name is not None and self.sinks == 0.0:
+            raise ValueError(f"{prefix or 'attention'}: learned sink scores need a count of sinks")
+        self.sink_scores: torch.Tensor | None = None
+        self.value_mix = None if value_mix is None else dict(value_mix)
+        if self.value_mix is not None and head_norm is None:
+            raise ValueError(f"{prefix or 'attention'}: values are mixed by the store that norms every head")
+        self.mix_weight = 0.0
         self.names = {"q": "q_proj.weight", "k": "k_proj.weight", "v": "v_proj.weight", "o": "o_proj.weight",
                       "q_norm": "q_norm.weight", "k_norm": "k_norm.weight", **(names or {})}
         self.q_size = self.num_heads * self.head_dim
@@ -154,6 +169,10 @@ class GroupedQueryAttention(Mixer):
             init = "zeros" if self.span_norm_offset == 1.0 else "ones"
             specs[self.name(self.names["q_norm"])] = TensorSpec((self.q_size,), init=init)
             specs[self.name(self.names["k_norm"])] = TensorSpec((self.kv_size,), init=init)
+        if self.sink_name is not None:
+            specs[self.name(self.sink_name)] = TensorSpec((self.num_heads,), init="zeros")
+        if self.value_mix is not None and not self.value_mix.get("source"):
+            specs[self.name(self.value_mix["name"])] = TensorSpec(())
         specs.update(self.position.tensor_specs())
         return specs
 
@@ -177,6 +196,10 @@ class GroupedQueryAttention(Mixer):
         if self.head_norm_eps is not None or self.span_norm_eps is not None:
             self.q_gain = tensors[self.name(self.names["q_norm"])].contiguous()
             self.k_gain = tensors[self.name(self.names["k_norm"])].contiguous()
+        if self.sink_name is not None:
+            self.sink_scores = tensors[self.name(self.sink_name)].float().contiguous()
+        if self.value_mix is not None and not self.value_mix.get("source"):
+            self.mix_weight = float(tensors[self.name(self.value_mix["name"])].float().item())
         self.position.load(tensors)
 
     def forward(self, x: torch.Tensor, ctx, cache: PagedKVView) -> torch.Tensor:
@@ -189,6 +212,14 @@ class GroupedQueryAttention(Mixer):
             more["head_norm"] = (self.q_gain, self.k_gain, self.head_norm_eps, self.head_norm_offset)
         if self.span_norm_eps is not None:
             more["span_norm"] = (self.q_gain, self.k_gain, self.span_norm_eps, self.span_norm_offset)
+        if self.value_mix is not None:
+            key = ("value_mix", self.value_mix["key"])
+            if self.value_mix.get("source"):
+                kept = torch.empty((ctx.num_tokens, self.v_size), dtype=torch.float32, device=x.device)
+                ctx.carried[key] = kept
+                more["values"] = {"keep": kept}
+            else:
+                more["values"] = {"blend": (ctx.carried[key], self.mix_weight)}
         q, q_stride = self.position.encode_and_store(
             qkv, self.num_heads, self.num_kv_heads, self.head_dim, ctx, cache, **more
         )
@@ -207,7 +238,8 @@ class GroupedQueryAttention(Mixer):
         ops = self.runtime.ops
         table = ctx.block_tables[cache.group]
         slopes = self.position.score_slopes(self.num_heads)
-        fast = (slopes is None and self.value_dim == self.head_dim and self.chunk is None and self.sinks == 0.0
+        bias = self.position.score_bias_table(self.num_heads)
+        fast = (slopes is None and bias is None and self.value_dim == self.head_dim and self.chunk is None and self.sinks == 0.0
                 and ops.mfma_attention_supported(qkv.dtype, self.head_dim, cache.block_size))
         if fast:
             out = ops.rows_buffer(ctx.num_tokens, self.out_size, qkv.dtype, qkv.device)
@@ -233,8 +265,10 @@ class GroupedQueryAttention(Mixer):
             return out
         if ops.tiled_attention_supported(qkv.dtype, self.head_dim, self.value_dim, cache.block_size, q_stride):
             return tiled_attention(ops, qkv, q_stride, cache.k, cache.v, table, ctx, heads=self.num_heads, scale=self.scale,
-                                   window=self.window, chunk=self.chunk, sinks=self.sinks, slopes=slopes, softcap=self.softcap)
+                                   window=self.window, chunk=self.chunk, sinks=self.sinks, slopes=slopes, softcap=self.softcap,
+                                   sink_scores=self.sink_scores, distance_bias=bias)
         return ops.paged_attention_generic(
             qkv, q_stride, cache.k, cache.v, table, ctx.token_seq, ctx.positions,
             self.num_heads, self.scale, self.window, slopes, self.softcap, chunk=self.chunk, sinks=self.sinks,
+            sink_scores=self.sink_scores, distance_bias=bias,
         )

@@ -135,6 +135,10 @@ class ResidualStream:
     #: A second output that has not been added yet, ``[S, T, H]`` 32-bit partial sums: a block whose
     #: two parts both add to the stream leaves one here, and the next norm adds both in its pass.
     also: torch.Tensor | None = None
+    #: ``(gain [H], eps, scale)``: ``pending`` is normalised on its own before it is added, so what the
+    #: stream gets is ``scale * gain * pending / rms(pending)``, in 32-bit (a block with a norm behind
+    #: each part); the norm that adds ``pending`` does this in the same pass.
+    pending_norm: tuple | None = None
 
 
 # ---------------------------------------------------------------------------------------------
@@ -207,6 +211,11 @@ class Norm(Part):
         stream is left as it is."""
         raise NotImplementedError
 
+    def pending_rule(self, scale: float) -> tuple:
+        """This norm as the rule of a pending output (``ResidualStream.pending_norm``): ``(gain, eps,
+        scale)``, for a block that normalises a part's output before the residual sum."""
+        raise NotImplementedError(f"{type(self).__name__} cannot be applied to a pending output")
+
 
 class PositionEncoding(Part):
     """Encodes positions into the queries and keys of an attention mixer and stores the
@@ -239,6 +248,12 @@ class PositionEncoding(Part):
         slopes ``m`` on the device, for which the score of key ``j`` for the query at position
         ``p`` of head ``h`` gets ``m[h] * (j - p)`` added before the softmax; ``None``: no such
         bias.  The attention mixer hands them to a kernel that takes them."""
+        return None
+
+    def score_bias_table(self, num_heads: int) -> torch.Tensor | None:
+        """Or through a table by distance: ``[num_heads, L]`` 32-bit on the device, for which the score
+        of the key ``n`` positions back gets ``table[h, min(n, L - 1)]`` added before the softmax;
+        ``None``: no such bias."""
         return None
 
 

@@ -136,3 +136,75 @@ class ParallelBlock(Block):
             self.runtime.ops.stream_fold(stream.residual, mixed, self.runtime.dtype)
         stream.pending = self.feed_forward.forward(x, ctx)
         return stream
+
+
+@register_block("sandwich")
+class SandwichBlock(Block):
+    """``h += m * norm_a2(mixer(norm_a(h))); h += m * norm_b2(feed_forward(norm_b(h)))``: a norm before
+    and one behind each part, and a multiplier ``m`` (``residual_scale``) on what is added.
+
+    The norm behind a part is not a pass of its own: the part's output waits in ``stream.pending``
+    with the norm's rule beside it (``stream.pending_norm``), and the next norm that carries the
+    residual sum (this block's, the next block's or the head's) normalises it, scales it and adds it,
+    all in 32-bit, before it normalises the sum.  A block without a feed-forward
+    (``feed_forward=None``) is its first half alone.  The four norms' checkpoint names under the
+    block's prefix are ``mixer_norm_name``, ``mixer_post_name``, ``ff_norm_name``, ``ff_post_name``."""
+
+    def __init__(
+        self,
+        prefix: str,
+        runtime: Runtime,
+        *,
+        mixer: PartSpec,
+        feed_forward: PartSpec | None,
+        norm: PartSpec,
+        residual_scale: float = 1.0,
+        mixer_name: str = "mix",
+        ff_name: str = "mlp",
+        mixer_norm_name: str = "norm1",
+        mixer_post_name: str = "norm1b",
+        ff_norm_name: str = "norm2",
+        ff_post_name: str = "norm2b",
+    ) -> None:
+        super().__init__(prefix, runtime)
+        self.residual_scale = float(residual_scale)
+        self.mixer_norm = build_part("norm", norm, self.name(mixer_norm_name), runtime)
+        self.mixer = build_part("mixer", mixer, self.name(mixer_name), runtime)
+        self.mixer_post = build_part("norm", norm, self.name(mixer_post_name), runtime)
+        self.ff_norm = self.feed_forward = self.ff_post = None
+        if feed_forward is not None:
+            self.ff_norm = build_part("norm", norm, self.name(ff_norm_name), runtime)
+            self.feed_forward = build_part("feed_forward", feed_forward, self.name(ff_name), runtime)
+            self.ff_post = build_part("norm", norm, self.name(ff_post_name), runtime)
+
+    def parts(self) -> list[Part]:
+        first = [self.mixer_norm, self.mixer, self.mixer_post]
+        return first if self.feed_forward is None else [*first, self.ff_norm, self.feed_forward, self.ff_post]
+
+    def activation_bytes(self, tokens: int, itemsize: int) -> int:
+        """A norm's output stays alive while the part it feeds runs."""
+        first = self.mixer_norm.activation_bytes(tokens, itemsize) + self.mixer.activation_bytes(tokens, itemsize)
+        if self.feed_forward is None:
+            return first
+        return max(first, self.ff_norm.activation_bytes(tokens, itemsize) + self.feed_forward.activation_bytes(tokens, itemsize))
+
+    def tensor_specs(self) -> dict[str, TensorSpec]:
+        specs: dict[str, TensorSpec] = {}
+        for part in self.parts():
+            specs.update(part.tensor_specs())
+        return specs
+
+    def load(self, tensors: Mapping[str, torch.Tensor]) -> None:
+        for part in self.parts():
+            part.load(tensors)
+
+    def forward(self, stream: ResidualStream, ctx, cache: CacheView) -> ResidualStream:
+        x = self.mixer_norm.forward_residual(stream)
+        stream.pending = self.mixer.forward(x, ctx, cache)
+        stream.pending_norm = self.mixer_post.pending_rule(self.residual_scale)
+        if self.feed_forward is None:
+            return stream
+        x = self.ff_norm.forward_residual(stream)
+        stream.pending = self.feed_forward.forward(x, ctx)
+        stream.pending_norm = self.ff_post.pending_rule(self.residual_scale)
+        return stream

@@ -28,7 +28,11 @@ class LatentAttention(Mixer):
     The query matrix and the down-projection are held as one matrix (one product a step); the two
     up-projections are stacks over the heads, ``[H, C, D]`` (transposed at load) and ``[H, Dv, C]``,
     run by ``ops.per_head_rows``.  ``rotation`` is the ``PartSpec`` of a rotary encoding (its tables
-    are what this part reads; ``turned <= R`` elements are turned, the rest pass).  ``names``: tensor
+    are what this part reads; ``turned <= R`` elements are turned, the rest pass; pairs in halves or,
+    if the encoding says ``neighbours``, ``(2i, 2i + 1)``).  ``window``: a token sees itself and the
+    ``window - 1`` tokens before it.  ``gate_name``: a matrix ``[H, hidden]`` of that name makes one
+    number per head from the mixer's input, and the head's output is multiplied by its sigmoid
+    before the output matrix (its rows ride behind the fused matrix's).  ``names``: tensor
     names under the part's prefix of ``q, down, down_norm, up_k, up_v, o``."""
 
     def __init__(
@@ -46,6 +50,8 @@ class LatentAttention(Mixer):
         norm_eps: float,
         rotation: PartSpec,
         names: Mapping[str, str] | None = None,
+        window: int | None = None,
+        gate_name: str | None = None,
     ) -> None:
         super().__init__(prefix, runtime)
         self.hidden_size = int(hidden_size)
@@ -57,6 +63,10 @@ class LatentAttention(Mixer):
         self.scale = float(scale)
         self.norm_eps = float(norm_eps)
         self.wide = self.rank + self.rot_dim
+        self.window = None if window is None else int(window)
+        if self.window is not None and self.window < 1:
+            raise ValueError(f"{prefix or 'latent attention'}: a window of {self.window} tokens")
+        self.gate_name = gate_name
         if min(self.num_heads, self.head_dim, self.rot_dim, self.value_dim, self.rank) < 1 or self.num_heads > 1024:
             raise ValueError(f"{prefix or 'latent attention'}: sizes must be positive and the heads at most 1,024")
         if self.wide > 512:
@@ -74,7 +84,7 @@ class LatentAttention(Mixer):
         self.o_weight: torch.Tensor | None = None    # [hidden, H Dv]
 
     def cache_need(self) -> CacheNeed:
-        return PagedKV(1, self.wide, None, 0)
+        return PagedKV(1, self.wide, self.window, 0)
 
     def activation_bytes(self, tokens: int, itemsize: int) -> int:
         per_token = (self.q_size + self.wide + self.num_heads * (self.head_dim + 2 * self.wide + self.value_dim)) * itemsize
@@ -82,7 +92,9 @@ class LatentAttention(Mixer):
 
     def tensor_specs(self) -> dict[str, TensorSpec]:
         n = self.names
+        gate = {} if self.gate_name is None else {self.name(self.gate_name): TensorSpec((self.num_heads, self.hidden_size))}
         return {
+            **gate,
             self.name(n["q"]): TensorSpec((self.q_size, self.hidden_size)),
             self.name(n["down"]): TensorSpec((self.wide, self.hidden_size)),
             self.name(n["down_norm"]): TensorSpec((self.rank,), init="ones"),
@@ -93,7 +105,10 @@ class LatentAttention(Mixer):
 
     def load(self, tensors: Mapping[str, torch.Tensor]) -> None:
         n = self.names
-        self.fused = torch.cat([tensors[self.name(n["q"])], tensors[self.name(n["down"])]], dim=0).contiguous()
+        rows = [tensors[self.name(n["q"])], tensors[self.name(n["down"])]]
+        if self.gate_name is not None:
+            rows.append(tensors[self.name(self.gate_name)])
+        self.fused = torch.cat(rows, dim=0).contiguous()
         self.down_gain = tensors[self.name(n["down_norm"])].contiguous()
         up_k = tensors[self.name(n["up_k"])].view(self.num_heads, self.head_dim, self.rank)
         self.up_k = up_k.transpose(1, 2).contiguous()
@@ -108,21 +123,25 @@ class LatentAttention(Mixer):
         slots = ctx.slot_mapping[cache.group] if cache.writable else None
         q_plain, q_wide = ops.latent_store(
             proj, cache.k, self.down_gain, self.norm_eps, self.rotation.cos, self.rotation.sin, ctx.positions, slots,
-            self.num_heads, self.head_dim, self.rot_dim, self.rank, cache.block_size, ctx.max_context_len - 1, dtype)
+            self.num_heads, self.head_dim, self.rot_dim, self.rank, cache.block_size, ctx.max_context_len - 1, dtype,
+            neighbours=self.rotation.neighbours, tail=0 if self.gate_name is None else self.num_heads)
         # The plain query parts through the keys' up-projection: what they are against the latent itself.
         carried = ops.per_head_rows(q_plain, self.up_k)
         q_wide[:, :, : self.rank].copy_(carried.view(tokens, self.num_heads, self.rank))
         stride = self.num_heads * self.wide
         if ops.tiled_attention_supported(dtype, self.wide, self.rank, cache.block_size, stride, True):
             attended = tiled_attention(ops, q_wide.view(tokens, stride), stride, cache.k, None, ctx.block_tables[cache.group],
-                                       ctx, heads=self.num_heads, scale=self.scale, value_dim=self.rank)
+                                       ctx, heads=self.num_heads, scale=self.scale, value_dim=self.rank, window=self.window)
         else:
             attended = ops.paged_attention_generic(
                 q_wide.view(tokens, stride), stride, cache.k, None, ctx.block_tables[cache.group], ctx.token_seq,
-                ctx.positions, self.num_heads, self.scale, None, value_dim=self.rank)
+                ctx.positions, self.num_heads, self.scale, self.window, value_dim=self.rank)
         values = ops.per_head_rows(attended.view(tokens * self.num_heads, self.rank), self.up_v)
         heads_out = values.view(tokens, self.num_heads * self.value_dim)
-        if dtype != torch.float32:  # the products' 32-bit results, rounded once for the output matrix
+        if self.gate_name is not None:
+            # Every head's output times the sigmoid of its gate (the projection's last columns), rounded once.
+            heads_out = ops.head_gate(heads_out, proj, self.q_size + self.wide, self.num_heads, dtype)
+        elif dtype != torch.float32:  # the products' 32-bit results, rounded once for the output matrix
             rounded = ops.rows_buffer(tokens, self.num_heads * self.value_dim, dtype, x.device)
             rounded.copy_(heads_out)
             heads_out = rounded

@@ -54,3 +54,41 @@ class SwiGLU(FeedForward):
     def forward(self, x: torch.Tensor, ctx) -> torch.Tensor:
         ops = self.runtime.ops
         return ops.linear(ops.linear_swiglu(x, self.gate_up_weight, self.rule), self.down_weight, for_residual=True)
+
+
+@register_feed_forward("mlp")
+class ActivatedMLP(FeedForward):
+    """``down(act(up(x)))``: a feed-forward without a gate.  ``activation`` is one of
+    ``ops.ACTIVATIONS`` (``relu_squared``: ``max(z, 0)^2``; ``relu``; ``silu``; ``gelu_tanh``), applied in
+    32-bit to the first product's sums and rounded once.  ``names``: the two matrices' tensor names
+    under the part's prefix."""
+
+    def __init__(self, prefix: str, runtime: Runtime, *, hidden_size: int, intermediate_size: int, activation: str,
+                 names: tuple[str, str] = ("up_proj.weight", "down_proj.weight")) -> None:
+        super().__init__(prefix, runtime)
+        self.hidden_size = int(hidden_size)
+        self.intermediate_size = int(intermediate_size)
+        self.activation = str(activation)
+        self.up_name, self.down_name = names
+        self.up_weight: torch.Tensor | None = None
+        self.down_weight: torch.Tensor | None = None
+
+    def tensor_specs(self) -> dict[str, TensorSpec]:
+        return {
+            self.name(self.up_name): TensorSpec((self.intermediate_size, self.hidden_size)),
+            self.name(self.down_name): TensorSpec((self.hidden_size, self.intermediate_size)),
+        }
+
+    def activation_bytes(self, tokens: int, itemsize: int) -> int:
+        """The up projection, its activation and the down projection (32-bit: it is added to the
+        residual stream) of a step."""
+        return tokens * (2 * self.intermediate_size * itemsize + self.hidden_size * 4)
+
+    def load(self, tensors: Mapping[str, torch.Tensor]) -> None:
+        self.up_weight = tensors[self.name(self.up_name)].contiguous()
+        self.down_weight = tensors[self.name(self.down_name)].contiguous()
+
+    def forward(self, x: torch.Tensor, ctx) -> torch.Tensor:
+        ops = self.runtime.ops
+        hidden = ops.activate(ops.linear(x, self.up_weight), self.activation, x.dtype)
+        return ops.linear(hidden, self.down_weight, for_residual=True)

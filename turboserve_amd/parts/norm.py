@@ -47,7 +47,13 @@ class RMSNorm(Norm):
 
     def forward_residual(self, stream: ResidualStream, rows: torch.Tensor | None = None) -> torch.Tensor:
         y = self.runtime.ops.add_rmsnorm(stream.residual, stream.pending, self.weight, self.eps, rows,
-                                         gain_offset=self.gain_offset, one_rounding=self.one_rounding, also=stream.also)
+                                         gain_offset=self.gain_offset, one_rounding=self.one_rounding, also=stream.also,
+                                         pending_norm=stream.pending_norm)
         if rows is None:
-            stream.pending = stream.also = None
+            stream.pending = stream.also = stream.pending_norm = None
         return y
+
+    def pending_rule(self, scale: float) -> tuple:
+        if self.gain_offset != 0.0:
+            raise ValueError(f"{self.prefix}: a norm on a pending output takes its gain as stored (no offset)")
+        return (self.weight, self.eps, float(scale))

@@ -33,7 +33,7 @@ and one 2,048-token prompt), ``--shape 32b --batch 64 --fill-hbm`` (a cache pool
 free memory), ``--closed-loop C [--sampled]`` (the reference's serving profile driven offline: 256
 requests of 128..1,024 tokens in and 64..512 out, C in flight; the library's products run at a
 few step sizes that are all timed at start-up, about 70 s the first time), ``--attention-prefill T[,CTX]`` (the
-prefill attention kernel alone), ``--sample-kernel ROWS`` (the sampling kernel alone), ``--hbm-read`` (a kernel that only reads: what the memory gives), ``--only-prefill [TOKENS]`` (one prompt's prefill alone, 2,048 tokens or TOKENS), ``--designs [2k,4k]`` (the Sisisun design beside a Qwen2 model of equal layer sizes: prefill and decode; with ``--design kisadra`` the Kisadra design beside Sisisun), ``--kernel-shares TRACE.csv`` (no GPU: the per-kernel table of a
+prefill attention kernel alone), ``--sample-kernel ROWS`` (the sampling kernel alone), ``--hbm-read`` (a kernel that only reads: what the memory gives), ``--only-prefill [TOKENS]`` (one prompt's prefill alone, 2,048 tokens or TOKENS), ``--designs [2k,4k]`` (the Sisisun design beside a Qwen2 model of equal layer sizes: prefill and decode; with ``--design kisadra`` the Kisadra design beside Sisisun, with ``--design dovudra`` the Dovudra design beside Kisadra), ``--kernel-shares TRACE.csv`` (no GPU: the per-kernel table of a
 ``rocprofv3 --kernel-trace`` of any of these runs).
 """
 
@@ -124,8 +124,8 @@ def parse_args(argv: list[str] | None = None) -> argparse.Namespace:
                    help="prefill and decode of the Sisisun design (random weights) at layer sizes that resemble a real "
                         "model's (2k, 4k: the width), beside a Qwen2 model of the same width, heads, feed-forward and "
                         "number of layer runs; prints one JSON object and exits")
-    p.add_argument("--design", choices=["sisisun", "kisadra"], default="sisisun",
-                   help="which design --designs measures: sisisun beside Qwen2, or kisadra beside sisisun")
+    p.add_argument("--design", choices=["sisisun", "kisadra", "dovudra"], default="sisisun",
+                   help="which design --designs measures: sisisun beside Qwen2, kisadra beside sisisun, or dovudra beside kisadra")
     return p.parse_args(argv)
 
 
@@ -521,6 +521,29 @@ def kisadra_pair(size: str) -> tuple[dict, dict]:
     return kisadra, design_pair(size)[0]
 
 
+#: ``--designs --design dovudra``: the Dovudra configuration of a size (eight layers: five latent with a window longer
+#: than the prompt, three with distance biases, a sink and a window of 1,024 that mix their values; feed-forwards without
+#: a gate) beside a Kisadra configuration of the same mixers' sizes in the same order (latent without a window; chunks
+#: of 1,024), no loop, and gated feed-forwards two thirds as wide, so that both have the same parameters.
+def dovudra_pair(size: str) -> tuple[dict, dict]:
+    width, heads, kv, ff, rank = {"2k": (2048, 16, 4, 8192, 256), "4k": (4096, 32, 8, 14336, 384)}[size]
+    order = ["latent_attention", "attention", "latent_attention", "latent_attention", "attention", "latent_attention",
+             "latent_attention", "attention"]
+    latent = {"heads": heads, "dim": 128, "rot_dim": 64, "vdim": 128, "kv_rank": rank, "scale": 192 ** -0.5}
+    biased = {"heads": heads, "kv_heads": kv, "dim": 128, "vdim": 128, "scale": 128 ** -0.5, "bias_max": 1024, "bias_rows": 32,
+              "mask": {"size": 1024}, "v_mix": True}
+    turning = {"base": 10000.0, "dims": 64, "scaling": {"factor": 8.0, "original": 1024, "fast": 32.0, "slow": 1.0}}
+    mixers = {"latent_attention": dict(latent, mask={"size": 4096}, rot=turning), "attention": biased}
+    dovudra = {"architecture": "Dovudra", "vocab": 32000, "width": width, "norm": {"eps": 1e-6}, "residual_mult": 0.5,
+               "layers": [{"type": kind, "mixer": mixers[kind], "mlp": {"kind": "dense", "ff": ff * 3 // 2}} for kind in order]}
+    beside = {"latent_attention": dict(latent, rot={"base": 10000.0, "dims": 64}),
+              "attention": {"heads": heads, "kv_heads": kv, "dim": 128, "vdim": 128, "scale": 128 ** -0.5, "mask": {"size": 1024}}}
+    kisadra = {"architecture": "Kisadra", "vocab": 32000, "width": width, "norm": {"eps": 1e-6},
+               "layers": [{"type": kind, "mixer": beside[kind], "mlp": {"kind": "dense", "ff": ff}} for kind in order],
+               "loop": {"start": 0, "stop": 0, "times": 1}}
+    return dovudra, kisadra
+
+
 def mixer_work(mixer, batch: int, context: int, prompt: int) -> tuple[float, float]:
     """``(elements a decode step of `batch` requests at `context` tokens reads from the cache or state,
     multiply-adds x 2 of a prompt of `prompt` tokens inside the mixer beside its plain projections)``."""
@@ -528,13 +551,14 @@ def mixer_work(mixer, batch: int, context: int, prompt: int) -> tuple[float, flo
     if kind == "GatedLinearAttention":
         state = mixer.num_heads * mixer.head_dim * mixer.value_dim
         return batch * 2 * state * 2.0, 4.0 * prompt * state  # 32-bit state read and written: 2 x 2 run-dtype elements
+    window = getattr(mixer, "window", None) or 10 ** 9
     if kind == "LatentAttention":
-        seen = prompt * (prompt + 1) / 2
+        seen = sum(min(i + 1, window) for i in range(prompt))
         per_head = 2.0 * prompt * mixer.rank * (mixer.head_dim + mixer.value_dim)
-        return batch * context * mixer.wide, mixer.num_heads * (2.0 * seen * (mixer.wide + mixer.rank) + per_head)
+        return batch * min(context, window) * mixer.wide, mixer.num_heads * (2.0 * seen * (mixer.wide + mixer.rank) + per_head)
     chunk = getattr(mixer, "chunk", None) or 10 ** 9
-    seen = sum(i % chunk + 1 for i in range(prompt))
-    visible = (context - 1) % chunk + 1
+    seen = sum(min(i % chunk + 1, window) for i in range(prompt))
+    visible = min((context - 1) % chunk + 1, window)
     width = mixer.head_dim + mixer.value_dim
     return batch * visible * mixer.num_kv_heads * width, 2.0 * seen * mixer.num_heads * width
 
@@ -577,7 +601,9 @@ def run_designs(sizes: list[str], dtype_name: str, steps: int, warmup: int, desi
     for size in sizes:
         size, _, only = size.partition(":")  # "2k:qwen2": that design alone; "2k:qwen2:prefill": that phase alone (for profiles)
         only, _, phase = only.partition(":")
-        labels, pair = (("kisadra", "sisisun"), kisadra_pair(size)) if design == "kisadra" else (("sisisun", "qwen2"), design_pair(size))
+        labels, pair = {"dovudra": (("dovudra", "kisadra"), dovudra_pair), "kisadra": (("kisadra", "sisisun"), kisadra_pair),
+                        "sisisun": (("sisisun", "qwen2"), lambda s: design_pair(s))}[design]
+        pair = pair(size)
         for label, shape in zip(labels, pair):
             if only and only != label:
                 continue

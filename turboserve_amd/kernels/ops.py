@@ -1236,11 +1236,14 @@ class Ops:
                                                 heads, kv_heads, head_dim, value_dim, block_size, *rule, 0, 1, *tables, self.stream()),
                    "ts_attention_tiles")
         if num_decode_seqs > 0:
-            # Workgroups per (request, KV head): enough to give every compute unit one, no more than the
-            # keys have tiles of 64 (a chunk or window bounds what a token sees).
+            # Workgroups per (request, KV head): enough to fill the compute units (key rows of up to 128
+            # elements leave room for four workgroups on each), no more than the keys have tiles of 64 (a
+            # chunk or window bounds what a token sees; a window starts anywhere inside a tile).
             seen = max(1, min(max_decode_context, chunk or max_decode_context, window or max_decode_context))
+            key_tiles = -(-seen // 64) + (1 if window and window < max_decode_context else 0)
             head_tiles = kv_heads * (-(-(heads // kv_heads) // 64))
-            splits = max(1, min(-(-seen // 64), -(-self.compute_units // (num_decode_seqs * head_tiles)), 64))
+            room = (4 if head_dim <= 128 else 1) * self.compute_units
+            splits = max(1, min(key_tiles, -(-room // (num_decode_seqs * head_tiles)), 64))
             partial_o = partial_ml = None
             if splits > 1:
                 partial_o = torch.empty((num_decode_seqs, heads, splits, value_dim), dtype=torch.float32, device=q.device)

@@ -149,6 +149,8 @@ attention_tiles_kernel(uint16_t* __restrict__ out, float* __restrict__ partial_o
     bias_row[i] = distance_bias ? distance_bias + (size_t)(live ? row_head(r) : 0) * bias_len : nullptr;
     sink_at[i] = (sink_scores && live) ? sink_scores[row_head(r)] : 0.f;
   }
+  // (Key rows that hold their values have no variant with a bias: the launch refuses it.)
+  const bool biased = !VALUES_IN_KEYS && distance_bias != nullptr;
   fa_f32x4 o[VD];
 #pragma unroll
   for (int vt = 0; vt < VD; ++vt) o[vt] = fa_f32x4{0.f, 0.f, 0.f, 0.f};
@@ -246,6 +248,20 @@ attention_tiles_kernel(uint16_t* __restrict__ out, float* __restrict__ partial_o
     __syncthreads();
     if (tile + 1 < tile_end) fetch(tile + 1);  // in flight while this tile is computed
     const int key0 = tile * FA_KEYS;
+    // The biases of this lane's 16 scores, asked for in one stretch ahead of the first product, so
+    // that they arrive while it runs (asked for where they are added, each is waited for on its own).
+    float bias_of[4][4];
+    if (biased) {
+#pragma unroll
+      for (int ct = 0; ct < 4; ++ct) {
+        const int key = key0 + 16 * ct + r16;
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+          const bool seen = key >= low[i] && key <= pos[i];
+          bias_of[ct][i] = bias_row[i][seen ? min(pos[i] - key, bias_len - 1) : 0];
+        }
+      }
+    }
     // S = Q K^T: four tiles of 16 keys.
     fa_f32x4 s[4];
 #pragma unroll
@@ -278,7 +294,7 @@ attention_tiles_kernel(uint16_t* __restrict__ out, float* __restrict__ partial_o
       for (int i = 0; i < 4; ++i) {
         float v = fmaf(slope[i], (float)(key - pos[i]), s[ct][i] * rule.scale);
         const bool seen = key >= low[i] && key <= pos[i];
-        if (distance_bias) v += bias_row[i][seen ? min(pos[i] - key, bias_len - 1) : 0];
+        if (biased) v += bias_of[ct][i];
         v = seen ? v : -INFINITY;
         s[ct][i] = v;
         tile_max[i] = fmaxf(tile_max[i], v);
@@ -438,7 +454,7 @@ extern "C" int ts_attention_tiles(void* out, void* partial_o, void* partial_ml, 
   if (mode == 0 && (!tiles || splits != 1)) return TS_ERR_ARG;
   if (mode == 1 && splits > 1 && (!partial_o || !partial_ml)) return TS_ERR_ARG;
   if (mode < 0 || mode > 1 || splits < 1 || splits > FA_MAX_SPLITS) return TS_ERR_ARG;
-  if ((sink_scores && !(sinks > 0.f)) || (distance_bias && bias_len < 1)) return TS_ERR_ARG;
+  if ((sink_scores && !(sinks > 0.f)) || (distance_bias && (bias_len < 1 || !v_pages))) return TS_ERR_ARG;
   if (heads < 1 || kv_heads < 1 || heads % kv_heads != 0 || heads > 65535) return TS_ERR_SHAPE;
   if (dk < 8 || dk > 448 || dk % 8 != 0 || dv < 8 || dv > 384 || dv % 8 != 0 || block_size < 8 || block_size % 8 != 0)
     return TS_ERR_SHAPE;

@@ -1219,6 +1219,7 @@ class Ops:
             _check_pages(k_pages, v_pages, q.dtype, any_value_width=True)
             value_dim = v_pages.shape[2]
         _need(value_dim is not None and (v_pages is not None or value_dim <= head_dim), "values inside the keys are their first value_dim elements")
+        _need(distance_bias is None or v_pages is not None, "key rows that hold their values take no bias by distance")
         _need(self.tiled_attention_supported(q.dtype, head_dim, value_dim, block_size, q_stride, v_pages is None),
               "a geometry the tiled attention kernel does not take")
         _need(heads % kv_heads == 0 and q.is_contiguous() and q.numel() >= tokens * q_stride and q_stride >= heads * head_dim,

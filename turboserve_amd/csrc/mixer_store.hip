@@ -226,9 +226,47 @@ head_gate_kernel(T* __restrict__ out, const float* __restrict__ values, const P*
                  size_t split_stride, int width, int gate_at, int heads, int vdim) {
   const int t = blockIdx.x;
   const int per = heads * vdim;
-  for (int i = threadIdx.x; i < per; i += blockDim.x) {
+  for (int i = blockIdx.y * blockDim.x + threadIdx.x; i < per; i += gridDim.y * blockDim.x) {
     const float g = folded(proj + (size_t)t * width + gate_at + i / vdim, splits, split_stride);
     out[(size_t)t * per + i] = from_float<T>(values[(size_t)t * per + i] / (1.f + expf(-g)));
+  }
+}
+
+// The same, four elements of one head a thread (vdim a multiple of 4, 16-byte aligned rows).
+template <typename T, typename P>
+__global__ void __launch_bounds__(256)
+head_gate_vec4_kernel(T* __restrict__ out, const float* __restrict__ values, const P* __restrict__ proj, int splits,
+                      size_t split_stride, int width, int gate_at, int heads, int vdim) {
+  const int t = blockIdx.x;
+  const int per = heads * vdim;
+  const int i = 4 * (blockIdx.y * blockDim.x + threadIdx.x);
+  if (i >= per) return;
+  const float4 v = *reinterpret_cast<const float4*>(values + (size_t)t * per + i);
+  const float g = folded(proj + (size_t)t * width + gate_at + i / vdim, splits, split_stride);
+  const float d = 1.f + expf(-g);
+  T* to = out + (size_t)t * per + i;
+  if constexpr (std::is_same<T, float>::value) {
+    *reinterpret_cast<float4*>(to) = make_float4(v.x / d, v.y / d, v.z / d, v.w / d);
+  } else {
+    uint2 packed;
+    packed.x = (uint32_t)from_float<bf16_t>(v.x / d).bits | ((uint32_t)from_float<bf16_t>(v.y / d).bits << 16);
+    packed.y = (uint32_t)from_float<bf16_t>(v.z / d).bits | ((uint32_t)from_float<bf16_t>(v.w / d).bits << 16);
+    *reinterpret_cast<uint2*>(to) = packed;
+  }
+}
+
+template <typename T, typename P>
+static void launch_head_gate(void* out, const float* values, const void* proj, int splits, size_t split_stride, int tokens,
+                             int width, int gate_at, int heads, int vdim, hipStream_t stream) {
+  const int per = heads * vdim;
+  if (vdim % 4 == 0 && ((uintptr_t)out | (uintptr_t)values) % 16 == 0) {
+    const dim3 grid(tokens, (per / 4 + 255) / 256);
+    hipLaunchKernelGGL((head_gate_vec4_kernel<T, P>), grid, dim3(256), 0, stream, (T*)out, values, (const P*)proj, splits,
+                       split_stride, width, gate_at, heads, vdim);
+  } else {
+    const dim3 grid(tokens, (per + 1023) / 1024);
+    hipLaunchKernelGGL((head_gate_kernel<T, P>), grid, dim3(256), 0, stream, (T*)out, values, (const P*)proj, splits,
+                       split_stride, width, gate_at, heads, vdim);
   }
 }
 
@@ -237,13 +275,12 @@ extern "C" int ts_head_gate(void* out, const float* values, const void* proj, in
   if (tokens == 0) return TS_OK;
   if (!out || !values || !proj || heads < 1 || vdim < 1 || splits < 1 || gate_at < 0 || gate_at + heads > width)
     return TS_ERR_ARG;
-  const dim3 grid(tokens), block(256);
   if (dtype == TS_F32)
-    hipLaunchKernelGGL((head_gate_kernel<float, float>), grid, block, 0, stream, (float*)out, values, (const float*)proj, splits, (size_t)split_stride, width, gate_at, heads, vdim);
+    launch_head_gate<float, float>(out, values, proj, splits, (size_t)split_stride, tokens, width, gate_at, heads, vdim, stream);
   else if (dtype == TS_BF16 && in_f32)
-    hipLaunchKernelGGL((head_gate_kernel<bf16_t, float>), grid, block, 0, stream, (bf16_t*)out, values, (const float*)proj, splits, (size_t)split_stride, width, gate_at, heads, vdim);
+    launch_head_gate<bf16_t, float>(out, values, proj, splits, (size_t)split_stride, tokens, width, gate_at, heads, vdim, stream);
   else if (dtype == TS_BF16)
-    hipLaunchKernelGGL((head_gate_kernel<bf16_t, bf16_t>), grid, block, 0, stream, (bf16_t*)out, values, (const bf16_t*)proj, 1, (size_t)0, width, gate_at, heads, vdim);
+    launch_head_gate<bf16_t, bf16_t>(out, values, proj, 1, (size_t)0, tokens, width, gate_at, heads, vdim, stream);
   else
     return TS_ERR_DTYPE;
   return ts_launch_status();

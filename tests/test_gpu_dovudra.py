@@ -308,6 +308,8 @@ ALONE = {
     "latent": dt.layer(dt.latent(3, 16, 8, 12, 24, 21, base=100.0, stretch=(4.0, 32, 8.0, 1.0)), None),
     "latent_part_turned_no_window": dt.layer(dt.latent(2, 8, 12, 20, 9, None, turned=6, base=7.0, scale=0.6), None),
     "latent_matrix_cores": dt.layer(dt.latent(4, 32, 16, 24, 48, 37, base=5000.0, stretch=(2.0, 16, 4.0, 1.0)), None),
+    # A cached row (latent and rotated part) longer than any matrix-core attention kernel takes.
+    "latent_long_rows": dt.layer(dt.latent(2, 16, 16, 8, 584, 30, base=1000.0), None),
     "dense": dt.layer(dt.latent(1, 8, 4, 8, 8, 4), dt.dense(44)),
 }
 

@@ -23,7 +23,7 @@
 // bitwise independent of how the request was cut into steps and of the batch around it.
 #include "common.hpp"
 
-#define ATTN_MAX_DIM 512
+#define ATTN_MAX_DIM 1024
 #define ATTN_TILE 64
 
 template <typename T>

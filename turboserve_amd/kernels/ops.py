@@ -199,8 +199,10 @@ def _check_pages(k_pages: torch.Tensor, v_pages: torch.Tensor, dtype: torch.dtyp
           "value pages must be [NB, Hkv, D, BS] for key pages [NB, Hkv, BS, D]")
 
 
-#: Largest head size an attention kernel takes (the generic kernel's; the matrix-core kernels stop at 256).
+#: Largest head size the attention parts take (the store that norms heads holds one; the matrix-core kernels stop at 256).
 ATTENTION_MAX_HEAD_DIM = 512
+#: Longest key row and widest value the generic attention kernel takes (a layer that caches one row for all heads).
+ATTENTION_MAX_ROW = 1024
 
 
 def attention_geometry_error(num_heads: int, num_kv_heads: int, head_dim: int) -> str | None:
@@ -1133,13 +1135,13 @@ class Ops:
             _need(value_dim is not None and 1 <= value_dim <= k_pages.shape[3],
                   "values inside the keys are their first value_dim elements")
         _, kv_heads, block_size, head_dim = k_pages.shape
-        _need(value_dim <= ATTENTION_MAX_HEAD_DIM, f"values of {value_dim} elements are wider than the kernel takes")
+        _need(value_dim <= ATTENTION_MAX_ROW, f"values of {value_dim} elements are wider than the kernel takes")
         _need((chunk is None or chunk >= 1) and sinks >= 0.0, "a chunk is at least one position, sinks are not negative")
         tokens = positions.numel()
         _need(q.is_contiguous() and q.numel() >= tokens * q_stride and q_stride >= heads * head_dim,
               "q does not hold [T, q_stride] rows")
         _need(block_table.dim() == 2 and token_seq.numel() == tokens, "block_table [S, MB], token_seq [T]")
-        _need(1 <= kv_heads and heads % kv_heads == 0 and heads <= 65535 and 1 <= head_dim <= ATTENTION_MAX_HEAD_DIM,
+        _need(1 <= kv_heads and heads % kv_heads == 0 and heads <= 65535 and 1 <= head_dim <= ATTENTION_MAX_ROW,
               f"{heads} query heads on {kv_heads} KV heads of {head_dim} elements are outside what the kernel takes")
         out = self.rows_buffer(tokens, heads * value_dim, q.dtype, q.device)
         _check(self.core.ts_paged_attention_generic(

@@ -7,6 +7,7 @@ from collections.abc import Mapping
 
 import torch
 
+from turboserve_amd.kernels.ops import ATTENTION_MAX_ROW
 from turboserve_amd.parts.attention import tiled_attention
 from turboserve_amd.parts.base import CacheNeed, Mixer, PagedKV, PagedKVView, PartSpec, Runtime, TensorSpec
 from turboserve_amd.parts.registry import build_part, register_mixer
@@ -69,9 +70,9 @@ class LatentAttention(Mixer):
         self.gate_name = gate_name
         if min(self.num_heads, self.head_dim, self.rot_dim, self.value_dim, self.rank) < 1 or self.num_heads > 1024:
             raise ValueError(f"{prefix or 'latent attention'}: sizes must be positive and the heads at most 1,024")
-        if self.wide > 512:
-            raise ValueError(f"{prefix or 'latent attention'}: a cached row of {self.wide} elements is above the 512 the "
-                             "attention kernel takes")
+        if self.wide > ATTENTION_MAX_ROW:
+            raise ValueError(f"{prefix or 'latent attention'}: a cached row of {self.wide} elements is above the "
+                             f"{ATTENTION_MAX_ROW} the attention kernel takes")
         self.rotation = build_part("position_encoding", rotation, prefix, runtime)
         if not 2 <= self.rotation.head_dim <= self.rot_dim:
             raise ValueError(f"{prefix or 'latent attention'}: {self.rotation.head_dim} turned elements do not fit {self.rot_dim}")

@@ -1,6 +1,6 @@
 """Which cache each scheduled layer call has, and how calls with equal needs share a pool.
 
-Calls whose mixers need the same pages (same KV heads, key and value widths, window and chunk) form a *group*:
+Calls whose mixers need the same pages (same KV heads, key and value widths, window, chunk and kept first keys) form a *group*:
 one page pool, one block table per request, one device tensor holding every member's keys and
 values.  A model whose layers differ (all keys in some, a window in others) has several
 groups, each with pages of its own, so a windowed group can give pages back while the request
@@ -25,6 +25,7 @@ class PageGroup:
     entries: tuple[int, ...]  # schedule entries that own a unit in this group (one per unit: an entry may own several)
     value_dim: int | None = None
     chunk: int | None = None  # a token reads no key below its own chunk of this many positions
+    keep_first: int = 0  # the first keys of a request that are read behind a window too
 
     @property
     def value_width(self) -> int:
@@ -54,7 +55,7 @@ class CacheLayout:
 
         def unit_of(entry: int, need) -> tuple | None:
             if isinstance(need, PagedKV):
-                key = (need.num_kv_heads, need.head_dim, need.window, need.value_width, need.chunk)
+                key = (need.num_kv_heads, need.head_dim, need.window, need.value_width, need.chunk, need.keep_first if need.window is not None else 0)
                 if key not in keys:
                     keys.append(key)
                     members.append([])
@@ -75,7 +76,7 @@ class CacheLayout:
                 units.append(tuple(unit_of(entry, one) for one in need))
             else:
                 units.append(unit_of(entry, need))
-        groups = tuple(PageGroup(k[0], k[1], k[2], tuple(m), None if k[3] == k[1] else k[3], k[4]) for k, m in zip(keys, members))
+        groups = tuple(PageGroup(k[0], k[1], k[2], tuple(m), None if k[3] == k[1] else k[3], k[4], k[5]) for k, m in zip(keys, members))
         return cls(groups, tuple(states), tuple(units))
 
     @classmethod
@@ -87,6 +88,9 @@ class CacheLayout:
 
     def chunks(self) -> list[int | None]:
         return [group.chunk for group in self.groups]
+
+    def kept(self) -> list[int]:
+        return [group.keep_first for group in self.groups]
 
     def bytes_per_page(self, page_size: int, itemsize: int) -> list[int]:
         """Bytes one page of each group takes (keys and values of all members); for one group

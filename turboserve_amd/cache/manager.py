@@ -44,7 +44,7 @@ class RequestCache:
     num_tokens: int = 0  # tokens that have slots
     state_slot: int = -1
     state_is_fresh: bool = True  # the slot has not been zeroed on the device yet
-    released: list[int] = field(default_factory=list)  # per group, leading pages given back
+    released: list[int] = field(default_factory=list)  # per group, pages given back, counted from the first page that may go
 
 
 class CacheManager:
@@ -55,6 +55,7 @@ class CacheManager:
         page_size: int,
         num_state_slots: int,
         chunks: Sequence[int | None] | None = None,
+        kept: Sequence[int] | None = None,
     ) -> None:
         if page_size < 1 or page_size & (page_size - 1):
             raise ValueError(f"page_size must be a power of two, got {page_size}")
@@ -66,6 +67,11 @@ class CacheManager:
         self.chunks = [None] * len(self.windows) if chunks is None else list(chunks)
         if len(self.chunks) != len(self.windows):
             raise ValueError(f"{len(self.chunks)} chunk sizes for {len(self.windows)} groups")
+        #: Per group: the first keys of a request that every later token reads, also behind a window; the
+        #: pages that hold them are never given back while the request runs.
+        self.kept = [0] * len(self.windows) if kept is None else [int(n) for n in kept]
+        if len(self.kept) != len(self.windows) or any(n < 0 for n in self.kept):
+            raise ValueError(f"{self.kept} kept first keys for {len(self.windows)} groups")
         self.page_size = page_size
         self.pools = [PageAllocator(n, page_size) for n in counts]
         self.state_slots = StateSlotPool(num_state_slots)
@@ -96,7 +102,7 @@ class CacheManager:
         reach = [r for r in (self.windows[group], self.chunks[group]) if r is not None]
         if not reach:
             return pages
-        return min(pages, ceil_div(min(reach) - 1 + max_portion, self.page_size) + 1)
+        return min(pages, ceil_div(min(reach) - 1 + max_portion, self.page_size) + 1 + self._kept_pages(group))
 
     def fits_pool(self, total_tokens: int, max_portion: int) -> bool:
         """Whether the request could run if it had the pools to itself."""
@@ -129,9 +135,14 @@ class CacheManager:
         self._requests[request] = entry
         return entry
 
+    def _kept_pages(self, group: int) -> int:
+        """Leading pages of a request that hold kept first keys."""
+        return ceil_div(self.kept[group], self.page_size)
+
     def _releasable(self, entry: RequestCache, group: int, start: int) -> int:
-        """Leading logical pages no query at position ``>= start`` can see."""
-        return min(lowest_key_read(start, self.windows[group], self.chunks[group]) // self.page_size, len(entry.tables[group]))
+        """Logical pages behind the kept ones that no query at position ``>= start`` can see."""
+        below = min(lowest_key_read(start, self.windows[group], self.chunks[group]) // self.page_size, len(entry.tables[group]))
+        return max(0, below - self._kept_pages(group))
 
     def pages_short(self, request: Hashable, num_new: int) -> list[int]:
         """Per group, how many pages more than are free a portion of ``num_new`` tokens needs
@@ -164,7 +175,7 @@ class CacheManager:
         for g, pool in enumerate(self.pools):
             table = entry.tables[g]
             upto = self._releasable(entry, g, start)
-            for index in range(entry.released[g], upto):
+            for index in range(entry.released[g] + self._kept_pages(g), upto + self._kept_pages(g)):
                 pool.decref(table[index])
                 table[index] = PAD_PAGE
                 table.entry_changed(index)
@@ -223,7 +234,7 @@ class CacheManager:
                     raise RuntimeError(f"{request!r}: group {g} table does not cover {entry.num_tokens} tokens")
                 for index, page in enumerate(table):
                     if page == PAD_PAGE:
-                        if index >= entry.released[g]:
+                        if not self._kept_pages(g) <= index < entry.released[g] + self._kept_pages(g):
                             raise RuntimeError(f"{request!r}: group {g} page {index} is missing")
                         continue
                     held[page] = held.get(page, 0) + 1

@@ -50,9 +50,9 @@ def activation_headroom_bytes(model, scheduler: SchedulerConfig, itemsize: int) 
     return model.activation_bytes(scheduler.max_num_batched_tokens, scheduler.max_num_seqs, itemsize)
 
 
-def window_pages_needed(window: int, scheduler: SchedulerConfig) -> int:
+def window_pages_needed(window: int, scheduler: SchedulerConfig, keep_first: int = 0) -> int:
     per_request = ceil_div(window - 1 + scheduler.max_num_batched_tokens, scheduler.block_size) + 1
-    return per_request * scheduler.max_num_seqs
+    return (per_request + ceil_div(keep_first, scheduler.block_size)) * scheduler.max_num_seqs
 
 
 def size_cache(
@@ -71,12 +71,13 @@ def size_cache(
     page = scheduler.block_size
     per_page = layout.bytes_per_page(page, itemsize)
     windows = layout.windows()
+    kept = layout.kept()
     cap = None if max_model_len is None else ceil_div(max_model_len, page) * scheduler.max_num_seqs
 
     def clamp(group: int, count: int) -> int:
         count = min(count, MAX_SLOTS // page)  # slots (page * page size + offset) travel as int32
         if windows[group] is not None:
-            count = min(count, window_pages_needed(windows[group], scheduler))
+            count = min(count, window_pages_needed(windows[group], scheduler, kept[group]))
         if cap is not None:
             count = min(count, cap)
         return count
@@ -96,7 +97,7 @@ def size_cache(
     remaining = budget
     for g, window in enumerate(windows):
         if window is not None:
-            counts[g] = clamp(g, window_pages_needed(window, scheduler))
+            counts[g] = clamp(g, window_pages_needed(window, scheduler, kept[g]))
             remaining -= counts[g] * per_page[g]
     full = [g for g, window in enumerate(windows) if window is None]
     if full:

@@ -69,3 +69,8 @@ def _ensure_builtin() -> None:
         from turboserve_amd.models.dovudra import dovudra_plan
 
         register_architecture("Dovudra", DovudraConfig.from_dict, dovudra_plan)
+    if "Legavik" not in ARCHITECTURES:
+        from turboserve_amd.config.legavik_config import LegavikConfig
+        from turboserve_amd.models.legavik import legavik_plan
+
+        register_architecture("Legavik", LegavikConfig.from_dict, legavik_plan)

@@ -4,7 +4,8 @@
 // One wavefront per (token, query head).  The token at absolute position p of request s sees
 // the keys lo..p of that request, lo = max(0, p - window + 1) for a windowed layer and 0
 // otherwise (src/turboserve/engine/model/attention.py:139-148: keys <= ctx - q_len + j; the
-// window bound is this engine's); with chunk > 0 also lo >= (p / chunk) * chunk: a token sees its
+// window bound is this engine's), and with keep_first > 0 also the keys 0 .. keep_first - 1 that lie
+// below lo (the first tokens of a request stay visible behind a window, at their true positions); with chunk > 0 also lo >= (p / chunk) * chunk: a token sees its
 // own chunk of positions only, chunks counted from position 0 of the request.  sinks > 0 adds that
 // many keys of score 0 without a value to the softmax's denominator; with sink_scores [Hq] their score
 // is the head's entry instead of 0 (it is not scaled and gets no bias).  distance_bias [Hq, L] (32-bit)
@@ -35,7 +36,7 @@ paged_attention_generic_kernel(T* __restrict__ out, const T* __restrict__ q, lon
                                int heads, int kv_heads, int dim, int vdim, int block_size, float scale,
                                float softcap, int window, const float* __restrict__ slopes, int chunk, float sinks,
                                const float* __restrict__ sink_scores, const float* __restrict__ distance_bias,
-                               int bias_len) {
+                               int bias_len, int keep_first) {
   __shared__ float qs[ATTN_MAX_DIM];
   __shared__ float ps[ATTN_TILE];
   __shared__ long long rows[ATTN_TILE];  // per key of the tile: offset of its value column
@@ -68,9 +69,13 @@ paged_attention_generic_kernel(T* __restrict__ out, const T* __restrict__ q, lon
   float m_run = sinks > 0.f ? (sink_scores ? sink_scores[h] : 0.f) : -INFINITY;
   float l_run = sinks > 0.f ? sinks : 0.f;
 
-  for (int base = lo; base <= p; base += ATTN_TILE) {
+  // Two stretches of keys: the kept first ones below the window, then lo .. p.
+  const int kept = min(keep_first, lo);
+  for (int stretch = kept > 0 ? 0 : 1; stretch < 2; ++stretch) {
+  const int first = stretch == 0 ? 0 : lo, last = stretch == 0 ? kept - 1 : p;
+  for (int base = first; base <= last; base += ATTN_TILE) {
     const int key = base + lane;
-    const bool valid = key <= p;
+    const bool valid = key <= last;
     float score = -INFINITY;
     long long row = 0;
     if (valid) {
@@ -94,7 +99,7 @@ paged_attention_generic_kernel(T* __restrict__ out, const T* __restrict__ q, lon
     ps[lane] = prob;
     rows[lane] = row;
     __syncthreads();
-    const int count = (p - base + 1 < ATTN_TILE) ? p - base + 1 : ATTN_TILE;
+    const int count = (last - base + 1 < ATTN_TILE) ? last - base + 1 : ATTN_TILE;
 #pragma unroll
     for (int c = 0; c < CHUNKS; ++c) {
       const int d = lane + c * ATTN_TILE;
@@ -105,6 +110,7 @@ paged_attention_generic_kernel(T* __restrict__ out, const T* __restrict__ q, lon
         acc[c] = a;
       }
     }
+  }
   }
 
   T* orow = out + ((size_t)t * heads + h) * vdim;
@@ -127,8 +133,9 @@ extern "C" int ts_paged_attention_generic(void* out, const void* q, long q_strid
                                           int heads, int kv_heads, int dim, int vdim, int block_size,
                                           float scale, float softcap, int window, const float* slopes, int chunk,
                                           float sinks, const float* sink_scores, const float* distance_bias,
-                                          int bias_len, int dtype, hipStream_t stream) {
+                                          int bias_len, int keep_first, int dtype, hipStream_t stream) {
   if (tokens == 0) return TS_OK;
+  if (keep_first < 0 || (keep_first > 0 && chunk > 0)) return TS_ERR_ARG;
   if (!out || !q || !k_pages || !block_table || !token_seq || !positions) return TS_ERR_ARG;
   if (chunk < 0 || !(sinks >= 0.f) || (!v_pages && vdim > dim)) return TS_ERR_ARG;
   if ((sink_scores && !(sinks > 0.f)) || (distance_bias && bias_len < 1)) return TS_ERR_ARG;
@@ -137,9 +144,9 @@ extern "C" int ts_paged_attention_generic(void* out, const void* q, long q_strid
     return TS_ERR_SHAPE;
   dim3 grid(tokens, heads), block(ATTN_TILE);
   if (dtype == TS_F32)
-    hipLaunchKernelGGL(paged_attention_generic_kernel<float>, grid, block, 0, stream, (float*)out, (const float*)q, q_stride, (const float*)k_pages, (const float*)v_pages, block_table, table_width, token_seq, positions, heads, kv_heads, dim, vdim, block_size, scale, softcap, window, slopes, chunk, sinks, sink_scores, distance_bias, bias_len);
+    hipLaunchKernelGGL(paged_attention_generic_kernel<float>, grid, block, 0, stream, (float*)out, (const float*)q, q_stride, (const float*)k_pages, (const float*)v_pages, block_table, table_width, token_seq, positions, heads, kv_heads, dim, vdim, block_size, scale, softcap, window, slopes, chunk, sinks, sink_scores, distance_bias, bias_len, keep_first);
   else if (dtype == TS_BF16)
-    hipLaunchKernelGGL(paged_attention_generic_kernel<bf16_t>, grid, block, 0, stream, (bf16_t*)out, (const bf16_t*)q, q_stride, (const bf16_t*)k_pages, (const bf16_t*)v_pages, block_table, table_width, token_seq, positions, heads, kv_heads, dim, vdim, block_size, scale, softcap, window, slopes, chunk, sinks, sink_scores, distance_bias, bias_len);
+    hipLaunchKernelGGL(paged_attention_generic_kernel<bf16_t>, grid, block, 0, stream, (bf16_t*)out, (const bf16_t*)q, q_stride, (const bf16_t*)k_pages, (const bf16_t*)v_pages, block_table, table_width, token_seq, positions, heads, kv_heads, dim, vdim, block_size, scale, softcap, window, slopes, chunk, sinks, sink_scores, distance_bias, bias_len, keep_first);
   else
     return TS_ERR_DTYPE;
   return ts_launch_status();

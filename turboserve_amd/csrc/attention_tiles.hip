@@ -2,7 +2,8 @@
 // kernels do not take (bfloat16): keys and values of different widths, values that are the first
 // elements of the key rows themselves (a layer that caches one vector per token), a bias on the
 // scores that is linear in the distance or read from a table by the distance, chunks of positions, a
-// window, sinks in the softmax's denominator (of score 0, or of a score per head).  Same arithmetic as ts_paged_attention_generic: scores, bias, masks and softmax in
+// window (behind which the first `keep` tokens of a request may stay visible, at their true positions),
+// sinks in the softmax's denominator (of score 0, or of a score per head).  Same arithmetic as ts_paged_attention_generic: scores, bias, masks and softmax in
 // 32-bit; products of bfloat16 operands accumulated in 32-bit.
 //
 // A workgroup of four wavefronts owns 64 query rows and walks the keys they may see in tiles of 64:
@@ -34,6 +35,7 @@ struct FaRule {
   float sinks;
   int window;
   int chunk;
+  int keep;  // the keys 0 .. keep - 1 are seen also below the window's lower bound
 };
 
 // Sum and maximum over the 16 lanes that hold one row of an accumulator tile (a row of lanes for
@@ -115,12 +117,20 @@ attention_tiles_kernel(uint16_t* __restrict__ out, float* __restrict__ partial_o
   // of a shared-out walk its share of the tiles.
   const int p_first = row_position(0), p_last = row_position(tile_rows - 1);
   const int key_lo = fa_lowest(p_first, rule.window, rule.chunk);
-  int tile_begin = key_lo / FA_KEYS, tile_end = p_last / FA_KEYS + 1;
+  // The walk: the tiles of the kept first keys that lie below the window's tiles, then the window's.
+  // Walk index w is tile w below `kept_tiles`, and tile w + window_shift from there on.
+  const int window_begin = key_lo / FA_KEYS;
+  const int kept_tiles = min((rule.keep + FA_KEYS - 1) / FA_KEYS, window_begin);
+  const int window_shift = window_begin - kept_tiles;
+  int tile_begin = 0, tile_end = kept_tiles + p_last / FA_KEYS + 1 - window_begin;
   if (splits > 1) {
     const int per = (tile_end - tile_begin + splits - 1) / splits;
     tile_begin = tile_begin + (int)blockIdx.z * per;
     tile_end = min(tile_end, tile_begin + per);
   }
+  auto tile_of = [&](int w) { return w < kept_tiles ? w : w + window_shift; };
+  // Keys from this one on (rounded up to 8) up to key_lo may lie in pages that were given back.
+  const int keep_end = (rule.keep + 7) & ~7;
 
   // The wavefront's queries as first operands: row wave * 16 + r16, elements 32 kd + 8 group ..
   ts_u32x4 qf[KD];
@@ -192,7 +202,8 @@ attention_tiles_kernel(uint16_t* __restrict__ out, float* __restrict__ partial_o
 #pragma unroll
     for (int j = 0; j < K_MINE; ++j) {
       // Outside key_lo .. last: a live key again (its page may have been given back, or never taken); masked later.
-      const int key = max(min(key0 + max(k_key[j], 0), last_key), key_lo);
+      int key = min(key0 + max(k_key[j], 0), last_key);
+      if (key >= keep_end) key = max(key, key_lo);
       const int page = table[key >> block_shift];
       const uint16_t* src = k_pages + ((((size_t)page * kv_heads + kvh) << block_shift) + (key & block_mask)) * dk + k_at[j];
       k_reg[j] = k_key[j] >= 0 ? *reinterpret_cast<const ts_u32x4*>(src) : ts_u32x4{0u, 0u, 0u, 0u};
@@ -202,7 +213,8 @@ attention_tiles_kernel(uint16_t* __restrict__ out, float* __restrict__ partial_o
       for (int j = 0; j < V_MINE; ++j) {
         const int piece = tid + j * FA_THREADS;
         const int d = piece / (FA_KEYS / 8);
-        const int key = max(min(key0 + 8 * (piece % (FA_KEYS / 8)), last_key & ~7), key_lo & ~7);  // eight keys of one page
+        int key = min(key0 + 8 * (piece % (FA_KEYS / 8)), last_key & ~7);  // eight keys of one page
+        if (key >= keep_end) key = max(key, key_lo & ~7);
         const int page = table[key >> block_shift];
         const uint16_t* src = v_pages + ((((size_t)page * kv_heads + kvh) * dv + d) << block_shift) + (key & block_mask);
         v_reg[j] = piece < v_pieces ? *reinterpret_cast<const ts_u32x4*>(src) : ts_u32x4{0u, 0u, 0u, 0u};
@@ -241,13 +253,13 @@ attention_tiles_kernel(uint16_t* __restrict__ out, float* __restrict__ partial_o
   __syncthreads();
 
   uint16_t* my_p = ps + wave * 16 * P_ROW;
-  if (tile_begin < tile_end) fetch(tile_begin);
-  for (int tile = tile_begin; tile < tile_end; ++tile) {
+  if (tile_begin < tile_end) fetch(tile_of(tile_begin));
+  for (int walk = tile_begin; walk < tile_end; ++walk) {
     __syncthreads();  // everyone has read the tile before
     stage();
     __syncthreads();
-    if (tile + 1 < tile_end) fetch(tile + 1);  // in flight while this tile is computed
-    const int key0 = tile * FA_KEYS;
+    if (walk + 1 < tile_end) fetch(tile_of(walk + 1));  // in flight while this tile is computed
+    const int key0 = tile_of(walk) * FA_KEYS;
     // The biases of this lane's 16 scores, asked for in one stretch ahead of the first product, so
     // that they arrive while it runs (asked for where they are added, each is waited for on its own).
     float bias_of[4][4];
@@ -257,7 +269,7 @@ attention_tiles_kernel(uint16_t* __restrict__ out, float* __restrict__ partial_o
         const int key = key0 + 16 * ct + r16;
 #pragma unroll
         for (int i = 0; i < 4; ++i) {
-          const bool seen = key >= low[i] && key <= pos[i];
+          const bool seen = (key >= low[i] || key < rule.keep) && key <= pos[i];
           bias_of[ct][i] = bias_row[i][seen ? min(pos[i] - key, bias_len - 1) : 0];
         }
       }
@@ -293,7 +305,7 @@ attention_tiles_kernel(uint16_t* __restrict__ out, float* __restrict__ partial_o
 #pragma unroll
       for (int i = 0; i < 4; ++i) {
         float v = fmaf(slope[i], (float)(key - pos[i]), s[ct][i] * rule.scale);
-        const bool seen = key >= low[i] && key <= pos[i];
+        const bool seen = (key >= low[i] || key < rule.keep) && key <= pos[i];
         if (biased) v += bias_of[ct][i];
         v = seen ? v : -INFINITY;
         s[ct][i] = v;
@@ -448,8 +460,9 @@ extern "C" int ts_attention_tiles(void* out, void* partial_o, void* partial_ml, 
                                   int first_seq, int heads, int kv_heads, int dk, int dv, int block_size, float scale,
                                   float softcap, int window, int chunk, float sinks, const float* slopes, int mode,
                                   int splits, const float* sink_scores, const float* distance_bias, int bias_len,
-                                  hipStream_t stream) {
+                                  int keep_first, hipStream_t stream) {
   if (items == 0) return TS_OK;
+  if (keep_first < 0 || (keep_first > 0 && chunk > 0)) return TS_ERR_ARG;
   if (!out || !q || !k_pages || !block_table || !query_start_loc || !context_lens) return TS_ERR_ARG;
   if (mode == 0 && (!tiles || splits != 1)) return TS_ERR_ARG;
   if (mode == 1 && splits > 1 && (!partial_o || !partial_ml)) return TS_ERR_ARG;
@@ -462,7 +475,7 @@ extern "C" int ts_attention_tiles(void* out, void* partial_o, void* partial_ml, 
   if (block_size & (block_size - 1)) return TS_ERR_SHAPE;  // slots are taken apart by shift and mask
   if (v_pages && (dk > 384 || dv > 256)) return TS_ERR_SHAPE;  // the widest tiles are built for values inside the key rows
   if ((((uintptr_t)q | (uintptr_t)k_pages | (uintptr_t)v_pages) & 15) != 0 || (q_stride % 8) != 0) return TS_ERR_ARG;
-  const FaRule rule = {scale, softcap, sinks, window, chunk};
+  const FaRule rule = {scale, softcap, sinks, window, chunk, keep_first};
   const int group_heads = heads / kv_heads;
   if (mode == 0 && items > 65535) return TS_ERR_SHAPE;
   const dim3 grid = mode == 0 ? dim3(heads, items, 1) : dim3(items, kv_heads * ((group_heads + FA_ROWS - 1) / FA_ROWS), splits);

@@ -7,6 +7,7 @@
 //                        parts are turned by the position's angles, latent and rotated key go into
 //                        the key pages as one row, the queries are split for what follows;
 //   ts_head_gate         every head's output times the sigmoid of a gate column of the projection;
+//   ts_scaled_pair       a_scale * a + b_scale * b of two parts' outputs, 32-bit;
 //   ts_stream_fold       residual (+)= a part's output (a tensor of the run type or 32-bit partial sums);
 //   ts_stream_pair       [x | origin] of two 32-bit streams side by side, in the run type.
 //
@@ -220,28 +221,42 @@ extern "C" int ts_latent_store(void* q_plain, void* q_wide, const void* proj, in
 // the head's gate, which is column gate_at + h of the token's row of a projection (`width` columns; of
 // type T, or `splits` 32-bit partial sums).  32-bit arithmetic, one rounding.
 // ---------------------------------------------------------------------------------------------
-template <typename T, typename P>
+template <typename V>
+__device__ __forceinline__ float4 gate_values4(const V* at);
+template <>
+__device__ __forceinline__ float4 gate_values4<float>(const float* at) {
+  return *reinterpret_cast<const float4*>(at);
+}
+template <>
+__device__ __forceinline__ float4 gate_values4<bf16_t>(const bf16_t* at) {
+  const uint2 raw = *reinterpret_cast<const uint2*>(at);
+  return make_float4(__uint_as_float(raw.x << 16), __uint_as_float(raw.x & 0xffff0000u), __uint_as_float(raw.y << 16),
+                     __uint_as_float(raw.y & 0xffff0000u));
+}
+
+// V: the type of the values, 32-bit or the run's.
+template <typename T, typename P, typename V>
 __global__ void __launch_bounds__(256)
-head_gate_kernel(T* __restrict__ out, const float* __restrict__ values, const P* __restrict__ proj, int splits,
+head_gate_kernel(T* __restrict__ out, const V* __restrict__ values, const P* __restrict__ proj, int splits,
                  size_t split_stride, int width, int gate_at, int heads, int vdim) {
   const int t = blockIdx.x;
   const int per = heads * vdim;
   for (int i = blockIdx.y * blockDim.x + threadIdx.x; i < per; i += gridDim.y * blockDim.x) {
     const float g = folded(proj + (size_t)t * width + gate_at + i / vdim, splits, split_stride);
-    out[(size_t)t * per + i] = from_float<T>(values[(size_t)t * per + i] / (1.f + expf(-g)));
+    out[(size_t)t * per + i] = from_float<T>(to_float(values[(size_t)t * per + i]) / (1.f + expf(-g)));
   }
 }
 
 // The same, four elements of one head a thread (vdim a multiple of 4, 16-byte aligned rows).
-template <typename T, typename P>
+template <typename T, typename P, typename V>
 __global__ void __launch_bounds__(256)
-head_gate_vec4_kernel(T* __restrict__ out, const float* __restrict__ values, const P* __restrict__ proj, int splits,
+head_gate_vec4_kernel(T* __restrict__ out, const V* __restrict__ values, const P* __restrict__ proj, int splits,
                       size_t split_stride, int width, int gate_at, int heads, int vdim) {
   const int t = blockIdx.x;
   const int per = heads * vdim;
   const int i = 4 * (blockIdx.y * blockDim.x + threadIdx.x);
   if (i >= per) return;
-  const float4 v = *reinterpret_cast<const float4*>(values + (size_t)t * per + i);
+  const float4 v = gate_values4<V>(values + (size_t)t * per + i);
   const float g = folded(proj + (size_t)t * width + gate_at + i / vdim, splits, split_stride);
   const float d = 1.f + expf(-g);
   T* to = out + (size_t)t * per + i;
@@ -255,34 +270,70 @@ head_gate_vec4_kernel(T* __restrict__ out, const float* __restrict__ values, con
   }
 }
 
-template <typename T, typename P>
-static void launch_head_gate(void* out, const float* values, const void* proj, int splits, size_t split_stride, int tokens,
+template <typename T, typename P, typename V>
+static void launch_head_gate(void* out, const void* values, const void* proj, int splits, size_t split_stride, int tokens,
                              int width, int gate_at, int heads, int vdim, hipStream_t stream) {
   const int per = heads * vdim;
   if (vdim % 4 == 0 && ((uintptr_t)out | (uintptr_t)values) % 16 == 0) {
     const dim3 grid(tokens, (per / 4 + 255) / 256);
-    hipLaunchKernelGGL((head_gate_vec4_kernel<T, P>), grid, dim3(256), 0, stream, (T*)out, values, (const P*)proj, splits,
-                       split_stride, width, gate_at, heads, vdim);
+    hipLaunchKernelGGL((head_gate_vec4_kernel<T, P, V>), grid, dim3(256), 0, stream, (T*)out, (const V*)values, (const P*)proj,
+                       splits, split_stride, width, gate_at, heads, vdim);
   } else {
     const dim3 grid(tokens, (per + 1023) / 1024);
-    hipLaunchKernelGGL((head_gate_kernel<T, P>), grid, dim3(256), 0, stream, (T*)out, values, (const P*)proj, splits,
-                       split_stride, width, gate_at, heads, vdim);
+    hipLaunchKernelGGL((head_gate_kernel<T, P, V>), grid, dim3(256), 0, stream, (T*)out, (const V*)values, (const P*)proj,
+                       splits, split_stride, width, gate_at, heads, vdim);
   }
 }
 
-extern "C" int ts_head_gate(void* out, const float* values, const void* proj, int in_f32, int splits, long split_stride,
-                            int tokens, int width, int gate_at, int heads, int vdim, int dtype, hipStream_t stream) {
+// values_f32: the values are 32-bit (else of the run's type, as the attention kernels leave them).
+extern "C" int ts_head_gate(void* out, const void* values, int values_f32, const void* proj, int in_f32, int splits,
+                            long split_stride, int tokens, int width, int gate_at, int heads, int vdim, int dtype,
+                            hipStream_t stream) {
   if (tokens == 0) return TS_OK;
   if (!out || !values || !proj || heads < 1 || vdim < 1 || splits < 1 || gate_at < 0 || gate_at + heads > width)
     return TS_ERR_ARG;
   if (dtype == TS_F32)
-    launch_head_gate<float, float>(out, values, proj, splits, (size_t)split_stride, tokens, width, gate_at, heads, vdim, stream);
+    launch_head_gate<float, float, float>(out, values, proj, splits, (size_t)split_stride, tokens, width, gate_at, heads, vdim, stream);
+  else if (dtype == TS_BF16 && in_f32 && values_f32)
+    launch_head_gate<bf16_t, float, float>(out, values, proj, splits, (size_t)split_stride, tokens, width, gate_at, heads, vdim, stream);
   else if (dtype == TS_BF16 && in_f32)
-    launch_head_gate<bf16_t, float>(out, values, proj, splits, (size_t)split_stride, tokens, width, gate_at, heads, vdim, stream);
+    launch_head_gate<bf16_t, float, bf16_t>(out, values, proj, splits, (size_t)split_stride, tokens, width, gate_at, heads, vdim, stream);
+  else if (dtype == TS_BF16 && values_f32)
+    launch_head_gate<bf16_t, bf16_t, float>(out, values, proj, 1, (size_t)0, tokens, width, gate_at, heads, vdim, stream);
   else if (dtype == TS_BF16)
-    launch_head_gate<bf16_t, bf16_t>(out, values, proj, 1, (size_t)0, tokens, width, gate_at, heads, vdim, stream);
+    launch_head_gate<bf16_t, bf16_t, bf16_t>(out, values, proj, 1, (size_t)0, tokens, width, gate_at, heads, vdim, stream);
   else
     return TS_ERR_DTYPE;
+  return ts_launch_status();
+}
+
+// ---------------------------------------------------------------------------------------------
+// out[i] = a_scale * a[i] + b_scale * b[i] in 32-bit: two parts' outputs (each a tensor of the run type or
+// 32-bit partial sums) as one addend of the residual stream.
+// ---------------------------------------------------------------------------------------------
+template <typename A, typename B>
+__global__ void scaled_pair_kernel(float* __restrict__ out, const A* __restrict__ a, int a_splits, size_t a_stride, float a_scale,
+                                   const B* __restrict__ b, int b_splits, size_t b_stride, float b_scale, size_t total) {
+  const size_t idx = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
+  if (idx >= total) return;
+  out[idx] = fmaf(a_scale, folded(a + idx, a_splits, a_stride), b_scale * folded(b + idx, b_splits, b_stride));
+}
+
+extern "C" int ts_scaled_pair(float* out, const void* a, int a_f32, int a_splits, long a_stride, float a_scale, const void* b,
+                              int b_f32, int b_splits, long b_stride, float b_scale, long total, int dtype, hipStream_t stream) {
+  if (total == 0) return TS_OK;
+  if (!out || !a || !b || total < 0 || a_splits < 1 || b_splits < 1) return TS_ERR_ARG;
+  if (dtype != TS_F32 && dtype != TS_BF16) return TS_ERR_DTYPE;
+  const dim3 grid((unsigned)((total + 255) / 256)), block(256);
+  const bool wide_a = a_f32 || dtype == TS_F32, wide_b = b_f32 || dtype == TS_F32;
+#define SP_GO(A, B)                                                                                                  \
+  hipLaunchKernelGGL((scaled_pair_kernel<A, B>), grid, block, 0, stream, out, (const A*)a, a_splits, (size_t)a_stride, \
+                     a_scale, (const B*)b, b_splits, (size_t)b_stride, b_scale, (size_t)total)
+  if (wide_a && wide_b) SP_GO(float, float);
+  else if (wide_a) SP_GO(float, bf16_t);
+  else if (wide_b) SP_GO(bf16_t, float);
+  else SP_GO(bf16_t, bf16_t);
+#undef SP_GO
   return ts_launch_status();
 }
 

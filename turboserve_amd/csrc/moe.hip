@@ -29,7 +29,7 @@ __device__ __forceinline__ int wave_argmax(float value, int index, float& best) 
 __global__ void __launch_bounds__(TS_WAVE)
 moe_select_kernel(int* __restrict__ taken, float* __restrict__ weights, float* __restrict__ extra_gate,
                   const float* __restrict__ z, int stride, int experts, int top, int groups, int keep,
-                  float route_scale, int softmax, const float* __restrict__ correction, int normalise) {
+                  float route_scale, int softmax, const float* __restrict__ correction, int normalise, int mark_top) {
   __shared__ float weight_of[MOE_MAX_EXPERTS];  // s: what a taken expert is weighted with
   __shared__ float score[MOE_MAX_EXPERTS];      // c: what experts are chosen by
   __shared__ float mark[MOE_MAX_EXPERTS];   // per group
@@ -63,7 +63,7 @@ moe_select_kernel(int* __restrict__ taken, float* __restrict__ weights, float* _
         const float s = score[g * size + i];
         if (s > a) { b = a; a = s; } else if (s > b) { b = s; }
       }
-      mark[g] = size > 1 ? a + b : a;
+      mark[g] = (size > 1 && mark_top > 1) ? a + b : a;  // a group's mark: its two largest summed, or its largest
       open_group[g] = keep >= groups ? 1 : 0;
     }
   }
@@ -108,14 +108,14 @@ moe_select_kernel(int* __restrict__ taken, float* __restrict__ weights, float* _
 
 extern "C" int ts_moe_select(int* taken, float* weights, float* extra_gate, const float* z, int tokens, int stride,
                              int experts, int top, int groups, int keep, float route_scale, int softmax,
-                             const float* correction, int normalise, hipStream_t stream) {
+                             const float* correction, int normalise, int mark_top, hipStream_t stream) {
   if (tokens == 0) return TS_OK;
-  if (!taken || !weights || !z) return TS_ERR_ARG;
+  if (!taken || !weights || !z || mark_top < 1 || mark_top > 2) return TS_ERR_ARG;
   if (experts < 1 || experts > MOE_MAX_EXPERTS || top < 1 || top > MOE_MAX_TOP || groups < 1 || experts % groups != 0 ||
       keep < 1 || keep > groups || top > (experts / groups) * keep || stride < experts + (extra_gate ? 1 : 0))
     return TS_ERR_SHAPE;
   hipLaunchKernelGGL(moe_select_kernel, dim3(tokens), dim3(TS_WAVE), 0, stream, taken, weights, extra_gate, z, stride,
-                     experts, top, groups, keep, route_scale, softmax, correction, normalise);
+                     experts, top, groups, keep, route_scale, softmax, correction, normalise, mark_top);
   return ts_launch_status();
 }
 

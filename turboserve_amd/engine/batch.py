@@ -49,6 +49,7 @@ class StepLimits:
     num_pages: Sequence[int]
     windows: Sequence[int | None]
     chunks: Sequence[int | None] | None = None  # per group: a token reads no key below its own chunk
+    kept: Sequence[int] | None = None  # per group: the first keys of a request that are read behind a window too
     vocab_size: int | None = None
     num_state_slots: int | None = None  # slots 0 .. num_state_slots are valid (the last is the padding row)
 
@@ -286,6 +287,9 @@ def check_packed(data: np.ndarray, layout: StepLayout, entries: Sequence[StepEnt
             lowest_key = np.maximum(lowest_key, (np.maximum(first_position, 0) // chunk) * chunk)
         columns = np.arange(width, dtype=np.int64)[None, :]
         read = (columns >= (lowest_key // page_size)[:, None]) & (columns < (-(-contexts // page_size))[:, None])
+        kept = 0 if limits.kept is None else int(limits.kept[group])
+        if kept > 0:  # the pages of the kept first keys are read whatever the window's bound
+            read |= (columns < -(-kept // page_size)) & (columns < (-(-contexts // page_size))[:, None])
         missing = np.argwhere(read & (table < 0))
         if missing.size:
             row, col = (int(v) for v in missing[0])

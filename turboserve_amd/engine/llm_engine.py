@@ -125,7 +125,7 @@ class LLMEngine:
             if storage is None:
                 raise ValueError("an engine built around a stand-in runner needs its scheduler passed in")
             cache = CacheManager(storage.layout.windows(), storage.num_pages, sched_cfg.block_size, sched_cfg.max_num_seqs,
-                                 chunks=storage.layout.chunks())
+                                 chunks=storage.layout.chunks(), kept=storage.layout.kept())
             scheduler = Scheduler(sched_cfg, cache)
         self.scheduler = scheduler
         self.runner = runner if runner is not None else ModelRunner(model, storage)

@@ -48,7 +48,8 @@ class TraceReplayer:
         num_pages = -(-max_tokens // rounding) * (rounding // page_size)
         self.max_live = max_live
         self.storage = build_storage(self.model, num_pages, page_size, max_live)
-        self.manager = CacheManager(self.storage.layout.windows(), num_pages, page_size, max_live, chunks=self.storage.layout.chunks())
+        self.manager = CacheManager(self.storage.layout.windows(), num_pages, page_size, max_live, chunks=self.storage.layout.chunks(),
+                                    kept=self.storage.layout.kept())
         self.runner = ModelRunner(self.model, self.storage)
 
     def run_step(self, record: dict[str, Any]):

@@ -33,7 +33,7 @@ class ModelRunner:
         self.num_steps = 0
         #: What a checked step's page ids, slots, token ids and state slots must lie inside.
         self.limits = StepLimits(
-            num_pages=tuple(storage.num_pages), windows=tuple(self.layout.windows()), chunks=tuple(self.layout.chunks()),
+            num_pages=tuple(storage.num_pages), windows=tuple(self.layout.windows()), chunks=tuple(self.layout.chunks()), kept=tuple(self.layout.kept()),
             vocab_size=self.vocab_size, num_state_slots=storage.num_state_slots,
         )
         #: Steps of single tokens are replayed as HIP graphs (see ``decode_graph``), unless a part

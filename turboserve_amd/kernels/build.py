@@ -36,6 +36,9 @@ MODULES: dict[str, tuple[str, ...]] = {
         "head_norm_store.hip",
         "mixer_store.hip",
         "linear_state.hip",
+        "delta_state.hip",
+        "short_conv.hip",
+        "tanh_norm.hip",
         "moe.hip",
         "attention_generic.hip",
         "attention_tiles.hip",

@@ -70,22 +70,39 @@ _SIGNATURES: dict[str, dict[str, list]] = {
         "ts_patch_tokens": [c_void_p, c_void_p, c_void_p, c_int, c_int, c_void_p],
         "ts_paged_attention_generic": [c_void_p, c_void_p, c_long, c_void_p, c_void_p, c_void_p, c_int,
                                        c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_int, c_int,
-                                       c_float, c_float, c_int, c_void_p, c_int, c_float, c_void_p, c_void_p, c_int, c_int,
+                                       c_float, c_float, c_int, c_void_p, c_int, c_float, c_void_p, c_void_p, c_int, c_int, c_int,
                                        c_void_p],
         "ts_attention_tiles": [c_void_p, c_void_p, c_void_p, c_void_p, c_long, c_void_p, c_void_p, c_void_p, c_int, c_void_p,
                                c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_int, c_int, c_int, c_float, c_float, c_int,
-                               c_int, c_float, c_void_p, c_int, c_int, c_void_p, c_void_p, c_int, c_void_p],
+                               c_int, c_float, c_void_p, c_int, c_int, c_void_p, c_void_p, c_int, c_int, c_void_p],
         "ts_attention_tiles_combine": [c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_int, c_float,
                                        c_void_p, c_void_p],
         "ts_head_norm_store": [c_void_p, c_long, c_void_p, c_int, c_int, c_long, c_void_p, c_void_p, c_void_p, c_void_p,
                                c_float, c_float, c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_int, c_int, c_int,
-                               c_int, c_int, c_int, c_void_p, c_void_p, c_float, c_void_p],
+                               c_int, c_int, c_int, c_void_p, c_void_p, c_float, c_int, c_int, c_int, c_int, c_float, c_int,
+                               c_int, c_void_p],
         "ts_span_norm_store": [c_void_p, c_long, c_void_p, c_int, c_int, c_long, c_void_p, c_void_p, c_void_p, c_void_p,
                                c_float, c_float, c_void_p, c_int, c_int, c_int, c_int, c_int, c_int, c_int, c_void_p],
         "ts_latent_store": [c_void_p, c_void_p, c_void_p, c_int, c_int, c_long, c_void_p, c_void_p, c_float, c_void_p,
                             c_void_p, c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_int, c_int, c_int, c_int, c_int, c_int,
                             c_void_p],
-        "ts_head_gate": [c_void_p, c_void_p, c_void_p, c_int, c_int, c_long, c_int, c_int, c_int, c_int, c_int, c_int, c_void_p],
+        "ts_head_gate": [c_void_p, c_void_p, c_int, c_void_p, c_int, c_int, c_long, c_int, c_int, c_int, c_int, c_int, c_int,
+                         c_void_p],
+        "ts_scaled_pair": [c_void_p, c_void_p, c_int, c_int, c_long, c_float, c_void_p, c_int, c_int, c_long, c_float, c_long,
+                           c_int, c_void_p],
+        "ts_add_tanh_norm": [c_void_p, c_void_p, c_void_p, c_int, c_int, c_long, c_void_p, c_void_p, c_float, c_void_p, c_int,
+                             c_int, c_int, c_void_p, c_int, c_long, c_void_p],
+        "ts_tanh_cap": [c_void_p, c_long, c_float, c_void_p],
+        "ts_short_conv": [c_void_p, c_int, c_void_p, c_int, c_int, c_long, c_int, c_int, c_int, c_void_p, c_int, c_void_p,
+                          c_void_p, c_void_p, c_void_p, c_int, c_int, c_int, c_void_p],
+        "ts_short_conv_carry": [c_void_p, c_void_p, c_int, c_int, c_long, c_int, c_int, c_int, c_int, c_void_p, c_void_p,
+                                c_int, c_int, c_void_p],
+        "ts_delta_prepare": [c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_int, c_long, c_int, c_int,
+                             c_int, c_int, c_void_p, c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_int, c_int, c_void_p],
+        "ts_delta_scan": [c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_int,
+                          c_int, c_int, c_int, c_int, c_int, c_void_p],
+        "ts_delta_finish": [c_void_p, c_void_p, c_void_p, c_int, c_int, c_long, c_int, c_int, c_int, c_void_p, c_void_p,
+                            c_float, c_int, c_int, c_int, c_int, c_void_p],
         "ts_stream_fold": [c_void_p, c_void_p, c_int, c_int, c_long, c_long, c_int, c_int, c_void_p],
         "ts_stream_pair": [c_void_p, c_void_p, c_void_p, c_int, c_int, c_int, c_void_p],
         "ts_linear_state_scan": [c_void_p, c_void_p, c_int, c_int, c_long, c_void_p, c_void_p, c_float, c_void_p, c_void_p,
@@ -98,7 +115,7 @@ _SIGNATURES: dict[str, dict[str, list]] = {
         "ts_copy_f32": [c_void_p, c_void_p, c_long, c_void_p],
         "ts_stream_offset": [c_void_p, c_void_p, c_void_p, c_int, c_int, c_int, c_void_p],
         "ts_moe_select": [c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_int, c_int, c_float,
-                          c_int, c_void_p, c_int, c_void_p],
+                          c_int, c_void_p, c_int, c_int, c_void_p],
         "ts_moe_pair_rows": [c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_int, c_int, c_float,
                              c_float, c_float, c_float, c_int, c_void_p],
         "ts_moe_group": [c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_int, c_void_p],
@@ -650,6 +667,11 @@ class Ops:
         max_position: int = 0,
         keep_values: torch.Tensor | None = None,
         blend_values: tuple[torch.Tensor, float] | None = None,
+        normed: bool = False,
+        norm_after: bool = False,
+        values_are_keys: bool = False,
+        query_temperature: tuple[float, int] | None = None,
+        tail: int = 0,
     ) -> tuple[torch.Tensor, int]:
         """Per-head norm of the q and k heads of the fused projection ``[T, Hq D + Hkv D + Hkv Dv]``
         (``x * rsqrt(mean(x^2) + eps) * (gain_offset + gain)`` in 32-bit, the gain ``[D]`` shared by
@@ -659,12 +681,18 @@ class Ops:
         the tensor that holds the queries and its row stride, as :meth:`rope_store` does.
         ``keep_values [T, Hkv Dv]`` 32-bit receives the step's values as projected;
         ``blend_values = (other [T, Hkv Dv] 32-bit, w)`` stores ``(1 - w) v + w other`` instead of ``v``
-        (another layer's values of the same tokens mixed in, in 32-bit)."""
+        (another layer's values of the same tokens mixed in, in 32-bit).  ``normed``: the heads are divided
+        by their root mean square also without gains; ``norm_after``: the norm follows the rotation; tables
+        ``[capacity, R/2]`` with ``R < D`` turn the first ``R`` elements of a head only; ``values_are_keys``:
+        the projection is ``[T, Hq D + Hkv D]`` and the values are the key heads as projected;
+        ``query_temperature = (coef, every)``: a query at position ``p`` is multiplied by ``1 + coef ln(floor((p
+        + 1) / every) + 1)``; ``tail``: a row of the projection holds that many columns more behind the heads."""
         _gpu(proj, k_pages, v_pages, q_gain, k_gain, positions, slots, cos, sin, keep_values)
         _i32(positions, "positions")
         _i32(slots, "slots")
         tokens = positions.numel()
-        width = (heads + kv_heads) * head_dim + kv_heads * value_dim
+        width = (heads + kv_heads) * head_dim + (0 if values_are_keys else kv_heads * value_dim) + int(tail)
+        _need(not values_are_keys or value_dim == head_dim, "values that are the keys have the keys' size")
         run_dtype = dtype or proj.dtype
         if proj.dim() == 3:
             _need(dtype is not None, "partial sums need the run dtype")
@@ -676,9 +704,9 @@ class Ops:
                 _need(gain.shape == (head_dim,) and gain.dtype == run_dtype and gain.is_contiguous(),
                       "a gain must be [D] of the run dtype")
         if cos is not None:
-            _need(sin is not None and head_dim % 2 == 0 and cos.shape == sin.shape and cos.dim() == 2
-                  and cos.shape[1] == head_dim // 2 and cos.dtype == torch.float32 and sin.dtype == torch.float32
-                  and cos.is_contiguous() and sin.is_contiguous(), "cos/sin must be float32 [capacity, D/2]")
+            _need(sin is not None and cos.shape == sin.shape and cos.dim() == 2 and 1 <= cos.shape[1] <= head_dim // 2
+                  and cos.dtype == torch.float32 and sin.dtype == torch.float32
+                  and cos.is_contiguous() and sin.is_contiguous(), "cos/sin must be float32 [capacity, R/2], R <= D")
             _need(max_position < cos.shape[0], f"position {max_position} is beyond the rotary tables ({cos.shape[0]})")
         if slots is not None:
             _need(slots.numel() == tokens, "one slot per token")
@@ -692,6 +720,8 @@ class Ops:
         else:
             q_out, q_stride = proj, width
         other, weight = (None, 0.0) if blend_values is None else blend_values
+        coef, every = (0.0, 1) if query_temperature is None else query_temperature
+        _need(every >= 1, "the query temperature counts positions in stretches of at least one")
         for held in (keep_values, other):
             if held is not None:
                 _gpu(held)
@@ -701,7 +731,8 @@ class Ops:
             _ptr(q_out), q_stride, _ptr(proj), is_f32, splits, stride, _ptr(k_pages), _ptr(v_pages), _ptr(q_gain),
             _ptr(k_gain), float(eps), float(gain_offset), _ptr(cos), _ptr(sin), _ptr(positions), _ptr(slots), tokens,
             heads, kv_heads, head_dim, value_dim, block_size, dtype_code(run_dtype), _ptr(keep_values), _ptr(other),
-            float(weight), self.stream()), "ts_head_norm_store")
+            float(weight), 1 if normed else 0, 1 if norm_after else 0, 0 if cos is None else 2 * cos.shape[1],
+            1 if values_are_keys else 0, float(coef), int(every), int(tail), self.stream()), "ts_head_norm_store")
         return q_out, q_stride
 
     # -- stores and stream steps of other mixers ------------------------------------------------
@@ -719,7 +750,8 @@ class Ops:
         :meth:`rope_store` does."""
         _gpu(proj, k_pages, v_pages, q_gain, k_gain, slots)
         _i32(slots, "slots")
-        width = (heads + kv_heads) * head_dim + kv_heads * value_dim
+        width = (heads + kv_heads) * head_dim + (0 if values_are_keys else kv_heads * value_dim) + int(tail)
+        _need(not values_are_keys or value_dim == head_dim, "values that are the keys have the keys' size")
         run_dtype = dtype or proj.dtype
         if proj.dim() == 3:
             _need(dtype is not None, "partial sums need the run dtype")
@@ -784,17 +816,17 @@ class Ops:
         return q_plain, q_wide
 
     def head_gate(self, values: torch.Tensor, proj: torch.Tensor, gate_at: int, heads: int, dtype: torch.dtype) -> torch.Tensor:
-        """``[T, H Dv]`` of ``dtype``: head ``h``'s ``Dv`` elements of the 32-bit ``values [T, H Dv]`` times
+        """``[T, H Dv]`` of ``dtype``: head ``h``'s ``Dv`` elements of ``values [T, H Dv]`` (32-bit, or of ``dtype``) times
         ``sigmoid`` of column ``gate_at + h`` of the token's row of ``proj`` (a projection of the run
         dtype or its 32-bit partial sums), in 32-bit with one rounding."""
         _gpu(values, proj)
         tokens, width = proj.shape[-2], proj.shape[-1]
         is_f32, splits, stride = self._partials(proj, tokens, width, dtype, "projection")
-        _need(values.dtype == torch.float32 and values.is_contiguous() and values.dim() == 2 and values.shape[0] == tokens
+        _need(values.dtype in (torch.float32, dtype) and values.is_contiguous() and values.dim() == 2 and values.shape[0] == tokens
               and values.shape[1] % heads == 0 and 0 <= gate_at and gate_at + heads <= width,
-              "values must be float32 [T, H Dv] and the gates' columns inside the projection")
+              "values must be [T, H Dv], 32-bit or of the run dtype, and the gates' columns inside the projection")
         out = self.rows_buffer(tokens, values.shape[1], dtype, values.device)
-        _check(self.core.ts_head_gate(_ptr(out), _ptr(values), _ptr(proj), is_f32, splits, stride, tokens, width, gate_at,
+        _check(self.core.ts_head_gate(_ptr(out), _ptr(values), 1 if values.dtype == torch.float32 else 0, _ptr(proj), is_f32, splits, stride, tokens, width, gate_at,
                                       heads, values.shape[1] // heads, dtype_code(dtype), self.stream()), "ts_head_gate")
         return out
 
@@ -909,16 +941,143 @@ class Ops:
                "ts_linear_state_finish")
         return y
 
+    def scaled_pair(self, a: torch.Tensor, a_scale: float, b: torch.Tensor, b_scale: float, dtype: torch.dtype) -> torch.Tensor:
+        """``a_scale * a + b_scale * b`` in 32-bit as one partial sum ``[1, T, H]``: two parts' outputs (each
+        ``[T, H]`` of the run dtype or ``[S, T, H]`` 32-bit partial sums) as one addend of the residual stream."""
+        _gpu(a, b)
+        tokens, hidden = a.shape[-2], a.shape[-1]
+        a_f32, a_splits, a_stride = self._partials(a, tokens, hidden, dtype, "the first output")
+        b_f32, b_splits, b_stride = self._partials(b, tokens, hidden, dtype, "the second output")
+        out = torch.empty((1, tokens, hidden), dtype=torch.float32, device=a.device)
+        _check(self.core.ts_scaled_pair(_ptr(out), _ptr(a), a_f32, a_splits, a_stride, float(a_scale), _ptr(b), b_f32, b_splits,
+                                        b_stride, float(b_scale), tokens * hidden, dtype_code(dtype), self.stream()), "ts_scaled_pair")
+        return out
+
+    def add_tanh_norm(self, residual: torch.Tensor, pending: torch.Tensor | None, weight: torch.Tensor, bias: torch.Tensor,
+                      alpha: float, rows: torch.Tensor | None = None, *, also: torch.Tensor | None = None) -> torch.Tensor:
+        """``residual += pending (+ also)`` in 32-bit (in place) and ``tanh(alpha s) * weight + bias`` of the sum
+        ``s`` in ``weight``'s dtype, rounded once; with ``rows`` only those rows, and ``residual`` is left alone.
+        ``pending`` is ``[T, H]`` of the run dtype or ``[S, T, H]`` 32-bit partial sums, ``also`` partial sums."""
+        _gpu(residual, pending, weight, bias, rows, also)
+        _i32(rows, "rows")
+        _need(residual.dim() == 2 and residual.dtype == torch.float32 and residual.is_contiguous(),
+              "residual must be contiguous float32 [T, H]")
+        tokens, hidden = residual.shape
+        _need(weight.shape == (hidden,) and weight.is_contiguous() and bias.shape == (hidden,) and bias.is_contiguous()
+              and bias.dtype == weight.dtype, "weight and bias must be [H] of one dtype")
+        is_f32, splits, stride = (0, 1, 0)
+        if pending is not None:
+            is_f32, splits, stride = self._partials(pending, tokens, hidden, weight.dtype, "pending")
+        also_splits, also_stride = 0, 0
+        if also is not None:
+            _need(also.dim() == 3 and also.dtype == torch.float32 and also.is_contiguous() and also.shape[1:] == (tokens, hidden),
+                  "a second addend must be float32 partial sums [S, T, H]")
+            also_splits, also_stride = also.shape[0], tokens * hidden
+        out_rows = tokens if rows is None else rows.numel()
+        y = self.rows_buffer(out_rows, hidden, weight.dtype, residual.device)
+        _check(self.core.ts_add_tanh_norm(_ptr(y), _ptr(residual), _ptr(pending), is_f32, splits, stride, _ptr(weight), _ptr(bias),
+                                          float(alpha), _ptr(rows), out_rows, hidden, dtype_code(weight.dtype), _ptr(also),
+                                          also_splits, also_stride, self.stream()), "ts_add_tanh_norm")
+        return y
+
+    def tanh_cap(self, x: torch.Tensor, cap: float) -> torch.Tensor:
+        """``x <- cap * tanh(x / cap)`` in place over a contiguous 32-bit tensor."""
+        _gpu(x)
+        _need(x.dtype == torch.float32 and x.is_contiguous() and cap > 0.0, "a positive cap on contiguous float32 values")
+        _check(self.core.ts_tanh_cap(_ptr(x), x.numel(), float(cap), self.stream()), "ts_tanh_cap")
+        return x
+
+    def short_conv(self, proj: torch.Tensor, first_col: int, taps: torch.Tensor, state: torch.Tensor, state_slots: torch.Tensor,
+                   token_seq: torch.Tensor, query_start_loc: torch.Tensor, *, tokens: int, num_seqs: int, dtype: torch.dtype,
+                   silu: bool = False, out_float32: bool = False) -> torch.Tensor:
+        """A short causal convolution over time on the ``C`` columns of ``proj`` from ``first_col`` on (``taps [C,
+        K]``: ``y_t = sum_j taps[:, j] u_(t - K + 1 + j)``), continuing every request from the ``K - 1`` inputs its
+        state slot holds (``state [slots, max(K - 1, 1), C]`` 32-bit, oldest first) and leaving its last ``K - 1``
+        inputs there.  ``proj`` is ``[T, W]`` of the run dtype or 32-bit partial sums.  Returns ``[T, C]`` of the
+        run dtype (32-bit with ``out_float32``), through ``silu`` if asked."""
+        _gpu(proj, taps, state, state_slots, token_seq, query_start_loc)
+        _i32(state_slots, "state_slots")
+        _i32(token_seq, "token_seq")
+        _i32(query_start_loc, "query_start_loc")
+        width = proj.shape[-1]
+        is_f32, splits, stride = self._partials(proj, tokens, width, dtype, "projection")
+        channels, k = taps.shape
+        _need(taps.dtype == dtype and taps.is_contiguous() and 1 <= k <= 8 and 0 <= first_col and first_col + channels <= width,
+              "taps must be [C, K] of the run dtype, K up to 8, over columns of the projection")
+        _need(state.dtype == torch.float32 and state.is_contiguous() and state.dim() == 3
+              and state.shape[1:] == (max(k - 1, 1), channels), "the state must be float32 [slots, K - 1, C]")
+        _need(token_seq.numel() >= tokens and query_start_loc.numel() >= num_seqs + 1 and state_slots.numel() >= num_seqs,
+              "row ranges and slots of every request")
+        wide = out_float32 or dtype == torch.float32
+        out = torch.empty((tokens, channels), dtype=torch.float32, device=proj.device) if wide \
+            else self.rows_buffer(tokens, channels, dtype, proj.device)
+        code = dtype_code(dtype)
+        _check(self.core.ts_short_conv(_ptr(out), 1 if wide else 0, _ptr(proj), is_f32, splits, stride, width, first_col, channels,
+                                       _ptr(taps), k, _ptr(state), _ptr(state_slots), _ptr(token_seq), _ptr(query_start_loc),
+                                       tokens, 1 if silu else 0, code, self.stream()), "ts_short_conv")
+        _check(self.core.ts_short_conv_carry(_ptr(state), _ptr(proj), is_f32, splits, stride, width, first_col, channels, k,
+                                             _ptr(state_slots), _ptr(query_start_loc), num_seqs, code, self.stream()),
+               "ts_short_conv_carry")
+        return out
+
+    def delta_rule(self, u: torch.Tensor, proj: torch.Tensor, *, beta_at: int, decay_at: int, gate_at: int, a2: torch.Tensor,
+                   dt_bias: torch.Tensor, a_log: torch.Tensor, g2: torch.Tensor, gain: torch.Tensor, eps: float,
+                   state: torch.Tensor, state_slots: torch.Tensor, query_start_loc: torch.Tensor, tokens: int, num_seqs: int,
+                   heads: int, kv_heads: int, head_dim: int, value_dim: int, dtype: torch.dtype) -> torch.Tensor:
+        """The gated delta rule over a step: per head and request a 32-bit state ``S [D, Dv]`` (``state [slots, H,
+        D, Dv]``) that every token decays, corrects and reads: ``S <- diag(g) S; w = beta (v - S^T k); S <- S + k
+        w^T; o = S^T q``.  ``u [T, 2 G D + H Dv]`` (32-bit) holds the step's convolved ``q | k | v``; ``q`` and ``k``
+        are made unit vectors per head (``q`` also times ``D^-1/2``), ``g = exp(-exp(a_log) softplus(a2 . low +
+        dt_bias))`` with ``low`` the ``a2.shape[1]`` columns of ``proj`` from ``decay_at`` on, ``beta`` the sigmoid of
+        the ``H`` columns from ``beta_at`` on.  Every head's ``o`` is divided by its root mean square, multiplied
+        by ``gain [Dv]`` and by ``sigmoid(g2 . low')``, ``low'`` the ``g2.shape[1]`` columns from ``gate_at`` on.
+        Returns ``[T, H Dv]`` of ``dtype``."""
+        _gpu(u, proj, a2, dt_bias, a_log, g2, gain, state, state_slots, query_start_loc)
+        _i32(state_slots, "state_slots")
+        _i32(query_start_loc, "query_start_loc")
+        width = proj.shape[-1]
+        is_f32, splits, stride = self._partials(proj, tokens, width, dtype, "projection")
+        keys, values = kv_heads * head_dim, heads * value_dim
+        _need(u.dtype == torch.float32 and u.is_contiguous() and u.shape == (tokens, 2 * keys + values),
+              "the convolved q | k | v must be float32 [T, 2 G D + H Dv]")
+        _need(heads % kv_heads == 0 and 1 <= head_dim <= 256, "heads in equal shares of the key heads, up to 256 key channels")
+        _need(a2.dim() == 2 and a2.shape[0] == heads * head_dim and 1 <= a2.shape[1] <= 128 and a2.dtype == dtype and a2.is_contiguous()
+              and dt_bias.shape == (heads * head_dim,) and dt_bias.dtype == dtype and dt_bias.is_contiguous(),
+              "the decay's matrix must be [H D, R] with R up to 128 and its bias [H D], of the run dtype")
+        _need(g2.dim() == 2 and g2.shape[0] == values and 1 <= g2.shape[1] <= 128 and g2.dtype == dtype and g2.is_contiguous()
+              and gain.shape == (value_dim,) and gain.dtype == dtype and gain.is_contiguous(),
+              "the gate's matrix must be [H Dv, R] with R up to 128 and the gain [Dv], of the run dtype")
+        _need(a_log.shape == (heads,) and a_log.dtype == torch.float32 and a_log.is_contiguous(), "a_log must be float32 [H]")
+        _need(state.dtype == torch.float32 and state.is_contiguous() and state.shape[1:] == (heads, head_dim, value_dim),
+              "the state must be float32 [slots, H, D, Dv]")
+        device = u.device
+        qn = torch.empty((tokens, keys), dtype=torch.float32, device=device)
+        kn = torch.empty((tokens, keys), dtype=torch.float32, device=device)
+        decay = torch.empty((tokens, heads * head_dim), dtype=torch.float32, device=device)
+        beta = torch.empty((tokens, heads), dtype=torch.float32, device=device)
+        o = torch.empty((tokens, values), dtype=torch.float32, device=device)
+        code = dtype_code(dtype)
+        _check(self.core.ts_delta_prepare(_ptr(qn), _ptr(kn), _ptr(decay), _ptr(beta), _ptr(u), _ptr(proj), is_f32, splits, stride,
+                                          width, beta_at, decay_at, a2.shape[1], _ptr(a2), _ptr(dt_bias), _ptr(a_log), tokens,
+                                          heads, kv_heads, head_dim, value_dim, code, self.stream()), "ts_delta_prepare")
+        _check(self.core.ts_delta_scan(_ptr(o), _ptr(state), _ptr(qn), _ptr(kn), _ptr(decay), _ptr(beta), _ptr(u), _ptr(state_slots),
+                                       _ptr(query_start_loc), 0, num_seqs, heads, kv_heads, head_dim, value_dim, self.stream()),
+               "ts_delta_scan")
+        y = self.rows_buffer(tokens, values, dtype, device)
+        _check(self.core.ts_delta_finish(_ptr(y), _ptr(o), _ptr(proj), is_f32, splits, stride, width, gate_at, g2.shape[1], _ptr(g2),
+                                         _ptr(gain), float(eps), tokens, heads, value_dim, code, self.stream()), "ts_delta_finish")
+        return y
+
     # -- routed feed-forward --------------------------------------------------------------------
 
     def moe_route(self, x: torch.Tensor, router: torch.Tensor, *, top: int, groups: int, keep: int, scale: float,
                   experts: int | None = None, softmax: bool = False, correction: torch.Tensor | None = None,
-                  normalise: bool = True) -> tuple[torch.Tensor, torch.Tensor, torch.Tensor | None]:
+                  normalise: bool = True, mark_top: int = 2) -> tuple[torch.Tensor, torch.Tensor, torch.Tensor | None]:
         """The router of a routed feed-forward: ``z = x router^T`` by the engine's product with a
         32-bit result, then in 32-bit ``s = sigmoid(z)`` or, with ``softmax``, the softmax over the
         ``experts`` outputs; experts are chosen by ``c = s + correction`` (``correction [experts]``
         32-bit; none: ``c = s``): they form ``groups`` equal groups of neighbours, a group's mark is
-        the sum of its two largest ``c``, only the ``keep`` best groups' experts can be taken, the
+        the sum of its two largest ``c`` (``mark_top = 1``: its largest alone), only the ``keep`` best groups' experts can be taken, the
         ``top`` of them with the largest ``c`` are.  Returns ``(taken [T, top] int32, weights [T, top]
         float32, gate)``: weights are ``s / (sum of the taken s + 1e-20) * scale``, or ``s * scale``
         where ``normalise`` is off.  With ``experts`` one less than the rows of ``router``, the last
@@ -941,7 +1100,7 @@ class Ops:
         gate = torch.empty((tokens,), dtype=torch.float32, device=x.device) if router.shape[0] > experts else None
         _check(self.core.ts_moe_select(_ptr(taken), _ptr(weights), _ptr(gate), _ptr(z), tokens, z.stride(0), experts, top,
                                        groups, keep, float(scale), 1 if softmax else 0, _ptr(correction),
-                                       1 if normalise else 0, self.stream()), "ts_moe_select")
+                                       1 if normalise else 0, int(mark_top), self.stream()), "ts_moe_select")
         return taken, weights, gate
 
     def moe_pair_rows(self, rows: torch.Tensor, weight: torch.Tensor, taken: torch.Tensor | None, *, share: int,
@@ -1104,8 +1263,10 @@ class Ops:
         value_dim: int | None = None,
         sink_scores: torch.Tensor | None = None,
         distance_bias: torch.Tensor | None = None,
+        keep_first: int = 0,
     ) -> torch.Tensor:
-        """Attention of every token over the keys ``lo..position`` of its request.  With
+        """Attention of every token over the keys ``lo..position`` of its request (behind a window
+        also over the request's first ``keep_first`` keys).  With
         ``softcap = c > 0`` a scaled score ``s`` becomes ``c * tanh(s / c)``.  Values may have a
         width of their own (value pages ``[NB, Hkv, Dv, BS]``); the result is ``[T, heads * Dv]``.
 
@@ -1149,7 +1310,7 @@ class Ops:
             block_table.shape[1], _ptr(token_seq), _ptr(positions), tokens, heads, kv_heads, head_dim, value_dim,
             block_size, float(scale), float(softcap), int(window or 0), _ptr(slopes) if slopes is not None else None,
             int(chunk or 0), float(sinks), _ptr(sink_scores), _ptr(distance_bias),
-            0 if distance_bias is None else distance_bias.shape[1], dtype_code(q.dtype), self.stream()),
+            0 if distance_bias is None else distance_bias.shape[1], int(keep_first), dtype_code(q.dtype), self.stream()),
             "ts_paged_attention_generic")
         return out
 
@@ -1200,7 +1361,7 @@ class Ops:
                         num_decode_seqs: int, max_decode_context: int, window: int | None = None, chunk: int | None = None,
                         sinks: float = 0.0, slopes: torch.Tensor | None = None, softcap: float = 0.0,
                         value_dim: int | None = None, sink_scores: torch.Tensor | None = None,
-                        distance_bias: torch.Tensor | None = None) -> torch.Tensor:
+                        distance_bias: torch.Tensor | None = None, keep_first: int = 0) -> torch.Tensor:
         """What :meth:`paged_attention_generic` computes, for bfloat16, on the matrix cores: the
         requests that bring several tokens (the first ``num_prefill_seqs``) in tiles of 64 tokens by
         one head (``prefill_tiles``: int32 ``[n, 2]`` from :meth:`attention_tile_list`), the
@@ -1209,7 +1370,7 @@ class Ops:
         several workgroups.  Returns ``[T, heads * Dv]``."""
         _gpu(q, k_pages, v_pages, block_table, query_start_loc, context_lens, prefill_tiles, slopes)
         self._score_tables(heads, sinks, sink_scores, distance_bias)
-        tables = (_ptr(sink_scores), _ptr(distance_bias), 0 if distance_bias is None else distance_bias.shape[1])
+        tables = (_ptr(sink_scores), _ptr(distance_bias), 0 if distance_bias is None else distance_bias.shape[1], int(keep_first))
         _i32(block_table, "block_table")
         _i32(query_start_loc, "query_start_loc")
         _i32(context_lens, "context_lens")
@@ -1244,6 +1405,8 @@ class Ops:
             # chunk or window bounds what a token sees; a window starts anywhere inside a tile).
             seen = max(1, min(max_decode_context, chunk or max_decode_context, window or max_decode_context))
             key_tiles = -(-seen // 64) + (1 if window and window < max_decode_context else 0)
+            if window and window < max_decode_context:
+                key_tiles += -(-int(keep_first) // 64)
             head_tiles = kv_heads * (-(-(heads // kv_heads) // 64))
             room = (4 if head_dim <= 128 else 1) * self.compute_units
             splits = max(1, min(key_tiles, -(-room // (num_decode_seqs * head_tiles)), 64))

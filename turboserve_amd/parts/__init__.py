@@ -1,6 +1,6 @@
 """The parts a model is assembled from; importing this package registers the built-in kinds."""
 
-from turboserve_amd.parts import attention, block, ends, experts, latent, linear_state, mlp, norm, rope, stream  # noqa: F401  (registration)
+from turboserve_amd.parts import attention, block, delta, ends, experts, latent, linear_state, mlp, norm, pair, rope, stream  # noqa: F401  (registration)
 from turboserve_amd.parts.base import (  # noqa: F401
     Block,
     CacheNeed,

@@ -42,7 +42,7 @@ class TensorSpec:
     ``kind`` is ``"float"`` (converted to the run's dtype), ``"float_keep32"`` (a tensor the
     file stores in 32-bit stays 32-bit, anything else is converted to the run's dtype) or
     ``"int"`` (kept as int32).  ``init`` says how the random-weights mode fills it:
-    ``"normal"`` (N(0, std)), ``"ones"`` or ``"zeros"``.
+    ``"normal"`` (N(0, std)), ``"ones"``, ``"zeros"`` or ``"constant:<value>"``.
     """
 
     shape: tuple[int, ...]
@@ -57,13 +57,15 @@ class PagedKV:
     caches one vector per token and head, and the value pages have no room at all);
     ``window`` keys are ever read again (``None``: all of them); with ``chunk = C`` a token at
     position ``p`` reads no key below ``(p // C) * C``, so pages below the chunk of the next token are
-    never read again either."""
+    never read again either; with ``keep_first = n`` the first ``n`` keys of a request are read behind a
+    window too, so the pages that hold them stay."""
 
     num_kv_heads: int
     head_dim: int
     window: int | None = None
     value_dim: int | None = None
     chunk: int | None = None
+    keep_first: int = 0
 
     @property
     def value_width(self) -> int:
@@ -240,7 +242,9 @@ class PositionEncoding(Part):
         encoding that knows nothing of these is still usable by the mixers that do not):
         ``value_dim`` (values ``Dv`` wide, the projection being ``[T, Hq D + Hkv D + Hkv Dv]``) and
         ``head_norm = (q_gain [D], k_gain [D], eps, gain_offset)`` (every q and k head is divided
-        by its root mean square and multiplied by ``gain_offset + gain`` before the encoding)."""
+        by its root mean square and multiplied by ``gain_offset + gain`` before the encoding), ``shape``
+        (a mapping of what else the per-head store takes: ``normed`` without gains, ``norm_after`` the
+        encoding, ``values_are_keys``, ``query_temperature``, ``tail`` columns behind the heads)."""
         raise NotImplementedError
 
     def score_slopes(self, num_heads: int) -> torch.Tensor | None:

@@ -82,7 +82,8 @@ class NormLinearHead(Head):
     """A norm over the summed stream, then ``[V, H]`` without bias, at the wanted rows only
     (model.py:108, :237-244).  ``tied_to`` names the tensor of another part (the token table)
     that serves as the matrix; the checkpoint's own copy under this part's prefix is then not
-    read (the reference shares one parameter, model.py:139-142)."""
+    read (the reference shares one parameter, model.py:139-142).  ``softcap = c``: the scores ``z`` leave as
+    ``c tanh(z / c)``."""
 
     def __init__(
         self,
@@ -95,8 +96,12 @@ class NormLinearHead(Head):
         norm_prefix: str,
         tied_to: str | None,
         weight_name: str = "weight",
+        softcap: float = 0.0,
     ) -> None:
         super().__init__(prefix, runtime)
+        self.softcap = float(softcap)
+        if self.softcap < 0.0:
+            raise ValueError(f"a cap of {self.softcap} on the scores")
         self.own_weight_name = weight_name
         self.vocab_size = int(vocab_size)
         self.hidden_size = int(hidden_size)
@@ -128,7 +133,10 @@ class NormLinearHead(Head):
 
     def forward(self, stream: ResidualStream, rows: torch.Tensor) -> torch.Tensor:
         hidden = self.norm.forward_residual(stream, rows)
-        return self.runtime.ops.linear_float32_out(hidden, self.weight)
+        scores = self.runtime.ops.linear_float32_out(hidden, self.weight)
+        if self.softcap > 0.0:
+            scores = self.runtime.ops.tanh_cap(scores.contiguous(), self.softcap)
+        return scores
 
 
 def standard_ends(vocab_size: int, hidden_size: int, norm: PartSpec, *, tie_head: bool,

@@ -29,7 +29,8 @@ class RoutedExperts(FeedForward):
     added to ``s`` where experts are chosen, while the weights use ``s`` alone); ``normalise =
     False`` (weights ``s * route_scale``, not divided by their sum); ``identity = n`` (the router
     has ``experts + n`` outputs, and the last ``n`` stand for the token itself: such a pair
-    contributes ``w * x`` and has no matrices).
+    contributes ``w * x`` and has no matrices); ``group_mark = "max"`` (a group's mark is its largest
+    score alone, not the sum of its two largest).
 
     The experts' matrices are stacked at load: ``[E, 2 I, H]`` with rows alternating gate, up,
     and ``[E, H, I]``.  A step routes on the device, runs every (token, taken expert) pair
@@ -60,6 +61,7 @@ class RoutedExperts(FeedForward):
         correction_name: str | None = None,
         normalise: bool = True,
         identity: int = 0,
+        group_mark: str = "top2_sum",
     ) -> None:
         super().__init__(prefix, runtime)
         self.hidden_size = int(hidden_size)
@@ -85,6 +87,9 @@ class RoutedExperts(FeedForward):
             raise ValueError(f"{prefix}: the router's kernel takes up to 1,024 outputs and 32 per token")
         if router_scores not in ("sigmoid", "softmax"):
             raise ValueError(f"{prefix}: router scores {router_scores!r} are neither 'sigmoid' nor 'softmax'")
+        if group_mark not in ("top2_sum", "max"):
+            raise ValueError(f"{prefix}: a group's mark {group_mark!r} is neither 'top2_sum' nor 'max'")
+        self.mark_top = 2 if group_mark == "top2_sum" else 1
         self.softmax = router_scores == "softmax"
         self.correction_name = correction_name or None
         self.normalise = bool(normalise)
@@ -146,7 +151,7 @@ class RoutedExperts(FeedForward):
         ops = self.runtime.ops
         taken, weights, gate = ops.moe_route(x, self.router, top=self.top, groups=self.groups, keep=self.keep,
                                              scale=self.route_scale, experts=self.outputs, softmax=self.softmax,
-                                             correction=self.correction, normalise=self.normalise)
+                                             correction=self.correction, normalise=self.normalise, mark_top=self.mark_top)
         grouping = ops.moe_grouping(taken, self.experts, x.dtype, self.hidden_size, self.expert_size)
         units = ops.moe_expert_units(x, self.gate_up, taken, self.rule, grouping)
         outputs = ops.moe_expert_outputs(units, self.down, taken, grouping)

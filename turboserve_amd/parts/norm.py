@@ -57,3 +57,51 @@ class RMSNorm(Norm):
         if self.gain_offset != 0.0:
             raise ValueError(f"{self.prefix}: a norm on a pending output takes its gain as stored (no offset)")
         return (self.weight, self.eps, float(scale))
+
+
+@register_norm("tanh_norm")
+class TanhNorm(Norm):
+    """A norm that computes no mean or variance: ``tanh(alpha x) * weight + bias`` with a learned scalar
+    ``alpha`` and vectors ``weight``, ``bias`` of the row's size, in 32-bit with one rounding.  The fused form
+    also carries the residual sum, kept in 32-bit.  ``weight_name``: the weight's name under the part's
+    prefix (empty: the prefix itself); ``alpha_name`` and ``bias_name`` are appended to the weight's name."""
+
+    def __init__(self, prefix: str, runtime: Runtime, *, size: int, weight_name: str = "weight", alpha_name: str = "alpha",
+                 bias_name: str = "b", initial_alpha: float = 0.5) -> None:
+        super().__init__(prefix, runtime)
+        self.size = int(size)
+        self.weight_name, self.alpha_name, self.bias_name = weight_name, alpha_name, bias_name
+        self.initial_alpha = float(initial_alpha)
+        self.weight: torch.Tensor | None = None
+        self.bias: torch.Tensor | None = None
+        self.alpha = self.initial_alpha
+
+    def _beside(self, suffix: str) -> str:
+        return f"{self.name(self.weight_name)}.{suffix}"
+
+    def tensor_specs(self) -> dict[str, TensorSpec]:
+        return {
+            self.name(self.weight_name): TensorSpec((self.size,), init="ones"),
+            self._beside(self.bias_name): TensorSpec((self.size,), init="zeros"),
+            self._beside(self.alpha_name): TensorSpec((), init=f"constant:{self.initial_alpha}"),
+        }
+
+    def activation_bytes(self, tokens: int, itemsize: int) -> int:
+        return tokens * self.size * itemsize
+
+    def load(self, tensors: Mapping[str, torch.Tensor]) -> None:
+        self.weight = tensors[self.name(self.weight_name)].contiguous()
+        self.bias = tensors[self._beside(self.bias_name)].contiguous()
+        self.alpha = float(tensors[self._beside(self.alpha_name)].float().item())
+
+    def forward(self, x: torch.Tensor) -> torch.Tensor:
+        raise NotImplementedError(f"{self.prefix}: this norm runs where it carries the residual sum")
+
+    def forward_residual(self, stream: ResidualStream, rows: torch.Tensor | None = None) -> torch.Tensor:
+        if stream.pending_norm is not None:
+            raise ValueError(f"{self.prefix}: a pending output with a norm of its own is added by a norm with statistics")
+        y = self.runtime.ops.add_tanh_norm(stream.residual, stream.pending, self.weight, self.bias, self.alpha, rows,
+                                           also=stream.also)
+        if rows is None:
+            stream.pending = stream.also = None
+        return y

@@ -55,16 +55,18 @@ def exact_rotary_tables(capacity: int, freq: torch.Tensor, magnitude: float) -> 
 
 
 def normed_store(runtime: Runtime, qkv, num_heads, num_kv_heads, head_dim, value_dim, ctx, cache: PagedKVView, slots,
-                 head_norm: tuple | None, cos, sin, span_norm: tuple | None = None, values: Mapping | None = None):
+                 head_norm: tuple | None, cos, sin, span_norm: tuple | None = None, values: Mapping | None = None,
+                 shape: Mapping | None = None):
     """The store of a mixer that asked for more than an encoding alone does: a norm per q and k
     head (``head_norm = (q_gain, k_gain, eps, gain_offset)``) and values of a width of their own,
     with the rotation by ``cos``/``sin`` where given, all in one pass (``ops.head_norm_store``); or
     a norm over all q heads at once and all k heads at once (``span_norm``, the same four with
     gains of the projections' full sizes; ``ops.span_norm_store``, which rotates nothing).  ``values =
     {"keep": tensor}`` and/or ``{"blend": (tensor, weight)}``: the step's values as projected are left in
-    ``keep``, and what is stored is mixed with ``blend`` (``ops.head_norm_store``)."""
+    ``keep``, and what is stored is mixed with ``blend`` (``ops.head_norm_store``).  ``shape``: what else the
+    per-head store takes (``normed``, ``norm_after``, ``values_are_keys``, ``query_temperature``, ``tail``)."""
     if span_norm is not None:
-        if values:
+        if values or shape:
             raise ValueError("values are kept or mixed by the per-head store only")
         if head_norm is not None or cos is not None:
             raise ValueError("a norm over the whole projection goes with no per-head norm and no rotation")
@@ -76,7 +78,7 @@ def normed_store(runtime: Runtime, qkv, num_heads, num_kv_heads, head_dim, value
     return runtime.ops.head_norm_store(
         qkv, cache.k, cache.v, q_gain, k_gain, eps, ctx.positions, slots, num_heads, num_kv_heads, head_dim, value_dim,
         cache.block_size, runtime.dtype, gain_offset=gain_offset, cos=cos, sin=sin, max_position=ctx.max_context_len - 1,
-        keep_values=(values or {}).get("keep"), blend_values=(values or {}).get("blend"),
+        keep_values=(values or {}).get("keep"), blend_values=(values or {}).get("blend"), **dict(shape or {}),
     )
 
 
@@ -98,7 +100,8 @@ class RotaryEncoding(PositionEncoding):
     ``interpolation = {factor, original, fast, slow}`` stretches the slow frequencies
     (:func:`interpolated_frequencies`); ``exact`` (implied by it) makes the tables from 64-bit angles
     rounded once.  ``neighbours``: the pairs turned together are ``(2i, 2i + 1)``; only a part that
-    reads the tables itself (the latent layer's store) takes that."""
+    reads the tables itself (the latent layer's store) takes that.  ``head_dim`` may be smaller than the
+    heads it is applied to: their first ``head_dim`` elements are turned, the rest pass."""
 
     shareable = True
 
@@ -154,14 +157,18 @@ class RotaryEncoding(PositionEncoding):
 
     def encode_and_store(self, qkv, num_heads, num_kv_heads, head_dim, ctx, cache: PagedKVView, *,
                          value_dim: int | None = None, head_norm: tuple | None = None, span_norm: tuple | None = None,
-                         values: Mapping | None = None):
+                         values: Mapping | None = None, shape: Mapping | None = None):
         if self.neighbours:
             raise ValueError("the stores of whole heads turn the pairs (i, i + D/2) only")
+        if self.head_dim > head_dim:
+            raise ValueError(f"{self.head_dim} turned elements do not fit heads of {head_dim}")
         self.ensure_capacity(ctx.max_context_len)
         slots = ctx.slot_mapping[cache.group] if cache.writable else None
-        if head_norm is not None or span_norm is not None or values or (value_dim is not None and value_dim != head_dim):
+        # (Tables narrower than the heads turn the heads' first elements only: the per-head store takes that.)
+        if (head_norm is not None or span_norm is not None or values or shape or self.head_dim != head_dim
+                or (value_dim is not None and value_dim != head_dim)):
             return normed_store(self.runtime, qkv, num_heads, num_kv_heads, head_dim, value_dim or head_dim, ctx, cache,
-                                slots, head_norm, self.cos, self.sin, span_norm, values)
+                                slots, head_norm, self.cos, self.sin, span_norm, values, shape)
         return self.runtime.ops.rope_store(
             qkv, cache.k, cache.v, self.cos, self.sin, ctx.positions, slots,
             num_heads, num_kv_heads, head_dim, cache.block_size, ctx.max_context_len - 1, self.runtime.dtype,
@@ -179,11 +186,11 @@ class NoPositionEncoding(PositionEncoding):
 
     def encode_and_store(self, qkv, num_heads, num_kv_heads, head_dim, ctx, cache: PagedKVView, *,
                          value_dim: int | None = None, head_norm: tuple | None = None, span_norm: tuple | None = None,
-                         values: Mapping | None = None):
+                         values: Mapping | None = None, shape: Mapping | None = None):
         slots = ctx.slot_mapping[cache.group] if cache.writable else None
-        if head_norm is not None or span_norm is not None or values or (value_dim is not None and value_dim != head_dim):
+        if head_norm is not None or span_norm is not None or values or shape or (value_dim is not None and value_dim != head_dim):
             return normed_store(self.runtime, qkv, num_heads, num_kv_heads, head_dim, value_dim or head_dim, ctx, cache,
-                                slots, head_norm, None, None, span_norm, values)
+                                slots, head_norm, None, None, span_norm, values, shape)
         return self.runtime.ops.rope_store(
             qkv, cache.k, cache.v, None, None, ctx.positions, slots,
             num_heads, num_kv_heads, head_dim, cache.block_size, ctx.max_context_len - 1, self.runtime.dtype,

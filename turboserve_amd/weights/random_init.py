@@ -37,6 +37,17 @@ def describe_model(config_data: Mapping[str, Any]):
     return config, DecoderModel(arch.build_plan(config), runtime)
 
 
+def _constant(init: str) -> float | None:
+    """The value of an initialisation ``"ones"``, ``"zeros"`` or ``"constant:<value>"``; ``None`` for a random one."""
+    if init == "ones":
+        return 1.0
+    if init == "zeros":
+        return 0.0
+    if init.startswith("constant:"):
+        return float(init.split(":", 1)[1])
+    return None
+
+
 def _sized(name: str, spec: TensorSpec) -> None:
     if any(size < 0 for size in spec.shape):
         raise ValueError(f"{name}: the configuration leaves a size of {spec.shape} to the checkpoint; "
@@ -52,10 +63,8 @@ def draw_tensors(
         if spec.kind == "int":
             raise ValueError(f"{name}: integer tables have no random initialisation")
         _sized(name, spec)
-        if spec.init == "ones":
-            yield name, torch.ones(spec.shape, dtype=dtype)
-        elif spec.init == "zeros":
-            yield name, torch.zeros(spec.shape, dtype=dtype)
+        if _constant(spec.init) is not None:
+            yield name, torch.full(spec.shape, _constant(spec.init), dtype=dtype)
         else:
             values = torch.empty(spec.shape, dtype=torch.float32)
             values.normal_(0.0, std, generator=generator)
@@ -99,10 +108,8 @@ def random_tensors_on_device(model, seed: int, *, std: float = 0.02) -> None:
     def make(name: str) -> torch.Tensor:
         spec = specs[name]
         _sized(name, spec)
-        if spec.init == "ones":
-            return torch.ones(spec.shape, dtype=runtime.dtype, device=runtime.device)
-        if spec.init == "zeros":
-            return torch.zeros(spec.shape, dtype=runtime.dtype, device=runtime.device)
+        if _constant(spec.init) is not None:
+            return torch.full(spec.shape, _constant(spec.init), dtype=runtime.dtype, device=runtime.device)
         generator = torch.Generator(device=runtime.device)
         generator.manual_seed(int(seed) * 1_000_003 + places[name])
         values = torch.empty(spec.shape, dtype=runtime.dtype, device=runtime.device)

@@ -98,7 +98,7 @@ def softmax_heads(q, k, v, scale: float, mask: dict | None, gate: torch.Tensor) 
         g = head // (H // G)
         for i in range(T):
             seen = [j for j in range(i + 1) if sees(i, j, mask)]
-            scores = torch.stack([(q[i, head] @ k[j, g]) * scale for j in seen])
+            scores = (k[seen, g] @ q[i, head]) * scale
             out[i, head] = torch.softmax(scores, dim=0) @ v[seen, g] * gate[i, head]
     return out.reshape(T, -1)
 
@@ -126,7 +126,8 @@ def convolved_attention(prefix: str, sizes: dict, tensors: dict, h: torch.Tensor
     H, G, D, Dv = sizes["heads"], sizes["kv_heads"], sizes["dim"], sizes["vdim"]
 
     def project(name):
-        return short_conv(h @ tensors[f"{prefix}.{name}"].T + tensors[f"{prefix}.{name}.b"], tensors[f"{prefix}.{name}.conv"])
+        projected = h @ tensors[f"{prefix}.{name}"].T + tensors[f"{prefix}.{name}.b"]
+        return short_conv(projected, tensors[f"{prefix}.{name}.conv"]) if sizes.get("conv") else projected
 
     q, k, v = project("q").view(T, H, D), project("k").view(T, G, D), project("v").view(T, G, Dv)
     q = unit_rms(q, eps) * tensors[prefix + ".q.norm"]

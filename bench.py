@@ -33,7 +33,7 @@ and one 2,048-token prompt), ``--shape 32b --batch 64 --fill-hbm`` (a cache pool
 free memory), ``--closed-loop C [--sampled]`` (the reference's serving profile driven offline: 256
 requests of 128..1,024 tokens in and 64..512 out, C in flight; the library's products run at a
 few step sizes that are all timed at start-up, about 70 s the first time), ``--attention-prefill T[,CTX]`` (the
-prefill attention kernel alone), ``--sample-kernel ROWS`` (the sampling kernel alone), ``--hbm-read`` (a kernel that only reads: what the memory gives), ``--only-prefill [TOKENS]`` (one prompt's prefill alone, 2,048 tokens or TOKENS), ``--designs [2k,4k]`` (the Sisisun design beside a Qwen2 model of equal layer sizes: prefill and decode; with ``--design kisadra`` the Kisadra design beside Sisisun, with ``--design dovudra`` the Dovudra design beside Kisadra), ``--kernel-shares TRACE.csv`` (no GPU: the per-kernel table of a
+prefill attention kernel alone), ``--sample-kernel ROWS`` (the sampling kernel alone), ``--hbm-read`` (a kernel that only reads: what the memory gives), ``--only-prefill [TOKENS]`` (one prompt's prefill alone, 2,048 tokens or TOKENS), ``--designs [2k,4k]`` (the Sisisun design beside a Qwen2 model of equal layer sizes: prefill and decode; with ``--design kisadra`` the Kisadra design beside Sisisun, with ``--design dovudra`` the Dovudra design beside Kisadra, with ``--design legavik`` the Legavik design beside Kisadra), ``--kernel-shares TRACE.csv`` (no GPU: the per-kernel table of a
 ``rocprofv3 --kernel-trace`` of any of these runs).
 """
 
@@ -124,8 +124,9 @@ def parse_args(argv: list[str] | None = None) -> argparse.Namespace:
                    help="prefill and decode of the Sisisun design (random weights) at layer sizes that resemble a real "
                         "model's (2k, 4k: the width), beside a Qwen2 model of the same width, heads, feed-forward and "
                         "number of layer runs; prints one JSON object and exits")
-    p.add_argument("--design", choices=["sisisun", "kisadra", "dovudra"], default="sisisun",
-                   help="which design --designs measures: sisisun beside Qwen2, kisadra beside sisisun, or dovudra beside kisadra")
+    p.add_argument("--design", choices=["sisisun", "kisadra", "dovudra", "legavik"], default="sisisun",
+                   help="which design --designs measures: sisisun beside Qwen2, kisadra beside sisisun, dovudra beside kisadra, "
+                        "or legavik beside kisadra")
     return p.parse_args(argv)
 
 
@@ -544,10 +545,49 @@ def dovudra_pair(size: str) -> tuple[dict, dict]:
     return dovudra, kisadra
 
 
+#: ``--designs --design legavik``: the Legavik configuration of a size (six layers: four parallel ones of causal attention
+#: with a convolution beside the gated delta rule, two of attention whose values are its keys behind a window of 1,024 that
+#: keeps the first 64 tokens; routed experts everywhere) beside a Kisadra configuration of the same mixers' sizes: for
+#: every parallel layer a causal attention layer without a feed-forward and a gated-linear-attention layer with the routed
+#: one, for every windowed layer an attention layer with chunks of 1,024; the same experts.
+def legavik_pair(size: str) -> tuple[dict, dict]:
+    width, heads, kv, experts, top, expert_ff, rank = {"2k": (2048, 16, 4, 32, 4, 1024, 64), "4k": (4096, 32, 8, 64, 6, 1408, 128)}[size]
+    routed = {"kind": "moe", "expert": {"ff": expert_ff}, "router": {"experts": experts, "top": top, "groups": {"count": 8, "keep": 4}}}
+    pair = {"left": {"heads": heads, "kv_heads": kv, "dim": 128, "vdim": 128, "scale": 128 ** -0.5, "conv": 4,
+                     "q_temp": {"coef": 0.1, "every": 256}},
+            "right": {"heads": heads, "kv_heads": heads, "dim": 128, "vdim": 128, "conv": 4, "decay_rank": rank, "gate_rank": rank},
+            "left_scale": 0.7, "right_scale": 0.7}
+    keyed = {"heads": heads, "kv_heads": kv, "dim": 128, "vdim": 128, "scale": 128 ** -0.5, "mask": {"size": 1024, "keep_first": 64},
+             "rot": {"base": 10000.0, "dims": 64, "scaling": {"factor": 8.0, "original": 1024, "fast": 32.0, "slow": 1.0}}}
+    order = ["parallel", "attention", "parallel", "parallel", "attention", "parallel"]
+    legavik = {"architecture": "Legavik", "vocab": 32000, "width": width, "norm": {"eps": 1e-6}, "logit_softcap": 30.0,
+               "layers": [{"type": kind, "mixer": pair if kind == "parallel" else keyed, "mlp": routed} for kind in order]}
+    attention = {"heads": heads, "kv_heads": kv, "dim": 128, "vdim": 128, "scale": 128 ** -0.5}
+    beside_routed = {"kind": "moe", "expert": {"ff": expert_ff, "limit": 7.0}, "router": {"experts": experts, "top": top}}
+    layers = []
+    for kind in order:
+        if kind == "parallel":
+            layers.append({"type": "attention", "mixer": dict(attention, mask={"size": 1 << 20}), "mlp": None})
+            layers.append({"type": "gla", "mixer": {"heads": heads, "dim": 128, "vdim": 128, "tau": 16.0, "rank": rank}, "mlp": beside_routed})
+        else:
+            layers.append({"type": "attention", "mixer": dict(attention, mask={"size": 1024}), "mlp": beside_routed})
+    kisadra = {"architecture": "Kisadra", "vocab": 32000, "width": width, "norm": {"eps": 1e-6}, "layers": layers,
+               "loop": {"start": 0, "stop": 0, "times": 1}}
+    return legavik, kisadra
+
+
 def mixer_work(mixer, batch: int, context: int, prompt: int) -> tuple[float, float]:
     """``(elements a decode step of `batch` requests at `context` tokens reads from the cache or state,
     multiply-adds x 2 of a prompt of `prompt` tokens inside the mixer beside its plain projections)``."""
     kind = type(mixer).__name__
+    if kind == "MixerPair":
+        one, other = mixer_work(mixer.left, batch, context, prompt), mixer_work(mixer.right, batch, context, prompt)
+        return one[0] + other[0], one[1] + other[1]
+    if kind == "GatedDeltaRule":
+        # The 32-bit state read and written (2 x 2 run-dtype elements each) and the convolution's rows; per token
+        # the decay, two reads and a write of the state, 2 flops each.
+        state = mixer.num_heads * mixer.head_dim * mixer.value_dim
+        return batch * (2 * state * 2.0 + 4.0 * (mixer.taps - 1) * mixer.channels), 8.0 * prompt * state
     if kind == "GatedLinearAttention":
         state = mixer.num_heads * mixer.head_dim * mixer.value_dim
         return batch * 2 * state * 2.0, 4.0 * prompt * state  # 32-bit state read and written: 2 x 2 run-dtype elements
@@ -557,8 +597,9 @@ def mixer_work(mixer, batch: int, context: int, prompt: int) -> tuple[float, flo
         per_head = 2.0 * prompt * mixer.rank * (mixer.head_dim + mixer.value_dim)
         return batch * min(context, window) * mixer.wide, mixer.num_heads * (2.0 * seen * (mixer.wide + mixer.rank) + per_head)
     chunk = getattr(mixer, "chunk", None) or 10 ** 9
-    seen = sum(min(i % chunk + 1, window) for i in range(prompt))
-    visible = min((context - 1) % chunk + 1, window)
+    kept = getattr(mixer, "keep_first", 0)
+    seen = sum(min(i % chunk + 1, window + kept, i + 1) for i in range(prompt))
+    visible = min((context - 1) % chunk + 1, window + kept, context)
     width = mixer.head_dim + mixer.value_dim
     return batch * visible * mixer.num_kv_heads * width, 2.0 * seen * mixer.num_heads * width
 
@@ -601,7 +642,8 @@ def run_designs(sizes: list[str], dtype_name: str, steps: int, warmup: int, desi
     for size in sizes:
         size, _, only = size.partition(":")  # "2k:qwen2": that design alone; "2k:qwen2:prefill": that phase alone (for profiles)
         only, _, phase = only.partition(":")
-        labels, pair = {"dovudra": (("dovudra", "kisadra"), dovudra_pair), "kisadra": (("kisadra", "sisisun"), kisadra_pair),
+        labels, pair = {"legavik": (("legavik", "kisadra"), legavik_pair),
+                        "dovudra": (("dovudra", "kisadra"), dovudra_pair), "kisadra": (("kisadra", "sisisun"), kisadra_pair),
                         "sisisun": (("sisisun", "qwen2"), lambda s: design_pair(s))}[design]
         pair = pair(size)
         for label, shape in zip(labels, pair):

@@ -97,9 +97,9 @@ _SIGNATURES: dict[str, dict[str, list]] = {
                           c_void_p, c_void_p, c_void_p, c_int, c_int, c_int, c_void_p],
         "ts_short_conv_carry": [c_void_p, c_void_p, c_int, c_int, c_long, c_int, c_int, c_int, c_int, c_void_p, c_void_p,
                                 c_int, c_int, c_void_p],
-        "ts_delta_prepare": [c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_int, c_long, c_int, c_int,
+        "ts_delta_prepare": [c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_int, c_long, c_int, c_int,
                              c_int, c_int, c_void_p, c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_int, c_int, c_void_p],
-        "ts_delta_scan": [c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_int,
+        "ts_delta_scan": [c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_int,
                           c_int, c_int, c_int, c_int, c_int, c_void_p],
         "ts_delta_finish": [c_void_p, c_void_p, c_void_p, c_int, c_int, c_long, c_int, c_int, c_int, c_void_p, c_void_p,
                             c_float, c_int, c_int, c_int, c_int, c_void_p],
@@ -750,8 +750,7 @@ class Ops:
         :meth:`rope_store` does."""
         _gpu(proj, k_pages, v_pages, q_gain, k_gain, slots)
         _i32(slots, "slots")
-        width = (heads + kv_heads) * head_dim + (0 if values_are_keys else kv_heads * value_dim) + int(tail)
-        _need(not values_are_keys or value_dim == head_dim, "values that are the keys have the keys' size")
+        width = (heads + kv_heads) * head_dim + kv_heads * value_dim
         run_dtype = dtype or proj.dtype
         if proj.dim() == 3:
             _need(dtype is not None, "partial sums need the run dtype")
@@ -1053,14 +1052,15 @@ class Ops:
         device = u.device
         qn = torch.empty((tokens, keys), dtype=torch.float32, device=device)
         kn = torch.empty((tokens, keys), dtype=torch.float32, device=device)
+        kq = torch.empty((tokens, kv_heads), dtype=torch.float32, device=device)
         decay = torch.empty((tokens, heads * head_dim), dtype=torch.float32, device=device)
         beta = torch.empty((tokens, heads), dtype=torch.float32, device=device)
         o = torch.empty((tokens, values), dtype=torch.float32, device=device)
         code = dtype_code(dtype)
-        _check(self.core.ts_delta_prepare(_ptr(qn), _ptr(kn), _ptr(decay), _ptr(beta), _ptr(u), _ptr(proj), is_f32, splits, stride,
+        _check(self.core.ts_delta_prepare(_ptr(qn), _ptr(kn), _ptr(kq), _ptr(decay), _ptr(beta), _ptr(u), _ptr(proj), is_f32, splits, stride,
                                           width, beta_at, decay_at, a2.shape[1], _ptr(a2), _ptr(dt_bias), _ptr(a_log), tokens,
                                           heads, kv_heads, head_dim, value_dim, code, self.stream()), "ts_delta_prepare")
-        _check(self.core.ts_delta_scan(_ptr(o), _ptr(state), _ptr(qn), _ptr(kn), _ptr(decay), _ptr(beta), _ptr(u), _ptr(state_slots),
+        _check(self.core.ts_delta_scan(_ptr(o), _ptr(state), _ptr(qn), _ptr(kn), _ptr(kq), _ptr(decay), _ptr(beta), _ptr(u), _ptr(state_slots),
                                        _ptr(query_start_loc), 0, num_seqs, heads, kv_heads, head_dim, value_dim, self.stream()),
                "ts_delta_scan")
         y = self.rows_buffer(tokens, values, dtype, device)

@@ -224,7 +224,8 @@ def test_the_delta_rule_whole_and_in_pieces(ops, dtype, heads, kv_heads, dim, vd
                                dt_bias=on_device["dt"], a_log=on_device["a_log"], g2=on_device["g2"], gain=on_device["gain"], eps=eps,
                                state=state, state_slots=torch.tensor([slots[i] for i in live], dtype=torch.int32, device=DEV),
                                query_start_loc=torch.tensor(starts, dtype=torch.int32, device=DEV), tokens=u.shape[0],
-                               num_seqs=len(live), heads=heads, kv_heads=kv_heads, head_dim=dim, value_dim=vdim, dtype=dtype)
+                               num_seqs=len(live), heads=heads, kv_heads=kv_heads, head_dim=dim, value_dim=vdim, dtype=dtype,
+                               num_long_seqs=(turn % 3) % (len(live) + 1))
             for j, i in enumerate(live):
                 got[i][done[i]:done[i] + counts[i]] = y[starts[j]:starts[j + 1]].float().cpu()
                 done[i] += counts[i]

@@ -7,7 +7,7 @@
 // Three launches a step:
 //   ts_delta_prepare  per token: q and k of every key head made unit vectors and their product k . q, the
 //                     decays of every head from the low-rank input, beta;
-//   ts_delta_scan     per (request, head, 32 value columns): the request's tokens in order, the state
+//   ts_delta_scan     per (request, head, 8 or 32 value columns): the request's tokens in order, the state
 //                     from and to the request's slot;
 //   ts_delta_finish   per (token, head): o divided by its root mean square, times a gain [Dv] shared by
 //                     the heads, times sigmoid(g2 . low'), rounded once to the run's type.
@@ -16,9 +16,6 @@
 #include "common.hpp"
 
 #define DS_MAX_LOW 128
-#define DS_PARTS 8    // lanes that share a value column of the scan, each with a stretch of the state's rows
-#define DS_COLS 32    // value columns of a workgroup of the scan
-#define DS_BATCH 16   // tokens staged at a time
 
 template <typename P>
 __device__ __forceinline__ float ds_input(const P* p, int splits, size_t stride) {
@@ -85,20 +82,34 @@ delta_prepare_kernel(float* __restrict__ qn, float* __restrict__ kn, float* __re
   }
 }
 
-// NR: state rows a thread holds.  Eight neighbouring lanes share a value column; lane part p of them
-// holds rows p NR .. p NR + NR - 1 (rows from `dim` on are padding and stay zero).
-template <int NR>
+// NR: state rows a thread holds; BATCH: tokens staged at a time.  DS_PARTS (8 or 16) neighbouring lanes
+// share a value column; lane part p of them holds, of every stretch of 4 DS_PARTS rows, the four rows from
+// 4 p on, so that the lanes of a column read neighbouring 16-byte pieces of a staged vector (rows from `dim`
+// on are padding and stay zero); a workgroup owns DS_COLS columns.  A batch's k, q, decays, values, beta and k . q
+// travel global memory -> registers -> LDS; the loads of the next batch are in flight while this one is
+// walked, and LDS holds two batches so that one barrier a batch is enough.
+//
+// A token costs every wavefront the same chain of instructions whatever it owns, and every lane reads its
+// rows of k, q and the decays from LDS, so what bounds a long walk is how thinly the state is spread: 16
+// lanes a column and 8 columns a workgroup give a head of 128 x 128 to 16 workgroups of two wavefronts
+// (prompt portions); single tokens, which read and write the state once, take 8 lanes a column and 32
+// columns a workgroup, whose rows of the state are whole cache lines.
+template <int NR, int BATCH, int DS_PARTS, int DS_COLS>
 __global__ void __launch_bounds__(DS_PARTS * DS_COLS)
 delta_scan_kernel(float* __restrict__ o, float* __restrict__ state, const float* __restrict__ qn, const float* __restrict__ kn,
                   const float* __restrict__ kq, const float* __restrict__ decay, const float* __restrict__ beta,
                   const float* __restrict__ u, const int* __restrict__ state_slots, const int* __restrict__ query_start_loc,
                   int first_seq, int heads, int kv_heads, int dim, int vdim) {
   constexpr int ROWS = DS_PARTS * NR;
-  __shared__ __attribute__((aligned(16))) float ks[DS_BATCH][ROWS];
-  __shared__ __attribute__((aligned(16))) float qs[DS_BATCH][ROWS];
-  __shared__ __attribute__((aligned(16))) float gs[DS_BATCH][ROWS];
-  __shared__ float vs[DS_BATCH][DS_COLS];
-  __shared__ float bs[DS_BATCH], kqs[DS_BATCH];
+  constexpr int THREADS = DS_PARTS * DS_COLS;
+  constexpr int MINE = BATCH * ROWS / THREADS;          // elements of each of k, q, g a thread fetches
+  constexpr int MINE_V = BATCH * DS_COLS / THREADS > 0 ? BATCH * DS_COLS / THREADS : 1;
+  static_assert(BATCH * ROWS % THREADS == 0 && BATCH <= THREADS, "a batch is shared out evenly");
+  __shared__ __attribute__((aligned(16))) float ks[2][BATCH][ROWS];
+  __shared__ __attribute__((aligned(16))) float qs[2][BATCH][ROWS];
+  __shared__ __attribute__((aligned(16))) float gs[2][BATCH][ROWS];
+  __shared__ float vs[2][BATCH][DS_COLS];
+  __shared__ float bs[2][BATCH], kqs[2][BATCH];
   const int seq = first_seq + blockIdx.x, h = blockIdx.y;
   const int g = h / (heads / kv_heads);
   const int tid = threadIdx.x;
@@ -108,69 +119,138 @@ delta_scan_kernel(float* __restrict__ o, float* __restrict__ state, const float*
   const int row0 = query_start_loc[seq], count = query_start_loc[seq + 1] - row0;
   const size_t u_width = (size_t)2 * kv_heads * dim + (size_t)heads * vdim;
   float* held = state + ((size_t)state_slots[seq] * heads + h) * dim * vdim;
+  // Row of the state that element i of this lane's registers holds.
+  auto row_of = [&](int i) { return (i / 4) * (4 * DS_PARTS) + part * 4 + i % 4; };
   float s[NR];
 #pragma unroll
   for (int i = 0; i < NR; ++i) {
-    const int d = part * NR + i;
+    const int d = row_of(i);
     s[i] = (live && d < dim) ? held[(size_t)d * vdim + c] : 0.f;
   }
-  for (int base = 0; base < count; base += DS_BATCH) {
-    const int batch = min(DS_BATCH, count - base);
-    __syncthreads();  // the batch before has been read
-    for (int i = tid; i < batch * ROWS; i += blockDim.x) {
+  float pk[MINE], pq[MINE], pg[MINE], pv[MINE_V], pb = 0.f, pkq = 0.f;
+  auto fetch = [&](int base) __attribute__((always_inline)) {
+    const int batch = min(BATCH, count - base);
+#pragma unroll
+    for (int e = 0; e < MINE; ++e) {
+      const int i = tid + e * THREADS;
       const int j = i / ROWS, d = i % ROWS;
-      const size_t t = (size_t)(row0 + base + j);
-      const bool in = d < dim;
-      ks[j][d] = in ? kn[(t * kv_heads + g) * dim + d] : 0.f;
-      qs[j][d] = in ? qn[(t * kv_heads + g) * dim + d] : 0.f;
-      gs[j][d] = in ? decay[(t * heads + h) * dim + d] : 0.f;
+      const bool in = j < batch && d < dim;
+      const size_t t = (size_t)(row0 + base + (in ? j : 0));
+      const int dd = in ? d : 0;
+      const float a = kn[(t * kv_heads + g) * dim + dd], b = qn[(t * kv_heads + g) * dim + dd], cc = decay[(t * heads + h) * dim + dd];
+      pk[e] = in ? a : 0.f;
+      pq[e] = in ? b : 0.f;
+      pg[e] = in ? cc : 0.f;
     }
-    for (int i = tid; i < batch * DS_COLS; i += blockDim.x) {
+#pragma unroll
+    for (int e = 0; e < MINE_V; ++e) {
+      const int i = tid + e * THREADS;
       const int j = i / DS_COLS, cc = blockIdx.z * DS_COLS + i % DS_COLS;
-      vs[j][i % DS_COLS] = cc < vdim ? u[(size_t)(row0 + base + j) * u_width + (size_t)2 * kv_heads * dim + (size_t)h * vdim + cc] : 0.f;
+      const bool in = i < BATCH * DS_COLS && j < batch && cc < vdim;
+      const float a = u[(size_t)(row0 + base + (in ? j : 0)) * u_width + (size_t)2 * kv_heads * dim + (size_t)h * vdim + (in ? cc : 0)];
+      pv[e] = in ? a : 0.f;
     }
-    if (tid < batch) {
-      bs[tid] = beta[(size_t)(row0 + base + tid) * heads + h];
-      kqs[tid] = kq[(size_t)(row0 + base + tid) * kv_heads + g];
+    const bool mine = tid < batch;
+    const size_t t = (size_t)(row0 + base + (mine ? tid : 0));
+    const float a = beta[t * heads + h], b = kq[t * kv_heads + g];
+    pb = mine ? a : 0.f;
+    pkq = mine ? b : 0.f;
+  };
+  auto stage = [&](int buf) __attribute__((always_inline)) {
+#pragma unroll
+    for (int e = 0; e < MINE; ++e) {
+      const int i = tid + e * THREADS;
+      ks[buf][i / ROWS][i % ROWS] = pk[e];
+      qs[buf][i / ROWS][i % ROWS] = pq[e];
+      gs[buf][i / ROWS][i % ROWS] = pg[e];
     }
+#pragma unroll
+    for (int e = 0; e < MINE_V; ++e) {
+      const int i = tid + e * THREADS;
+      if (i < BATCH * DS_COLS) vs[buf][i / DS_COLS][i % DS_COLS] = pv[e];
+    }
+    if (tid < BATCH) {
+      bs[buf][tid] = pb;
+      kqs[buf][tid] = pkq;
+    }
+  };
+  if (count > 0) fetch(0);
+  int buf = 0;
+  float* o_at = o + ((size_t)row0 * heads + h) * vdim + c;  // this column's output of the token being walked
+  const size_t o_step = (size_t)heads * vdim;
+  constexpr int Q = NR / 4;
+  for (int base = 0; base < count; base += BATCH, buf ^= 1) {
+    const int batch = min(BATCH, count - base);
+    stage(buf);  // (the other buffer's readers were let go by the barrier of the batch before)
     __syncthreads();
+    // In flight while this batch is walked; asked for unconditionally (behind the last batch: the last
+    // token again, which nobody stages), so that no wait for it is placed inside the walk.
+    fetch(min(base + BATCH, count - 1));
+    // A token's vectors are read from LDS while the token before it is walked.
+    float4 kk[Q], qq[Q], gg[Q], nk[Q], nq[Q], ng[Q];
+    float vv, bb, kqv, nv, nb, nkq;
+    auto read = [&](int j, float4* k4, float4* q4, float4* g4, float& v1, float& b1, float& kq1) __attribute__((always_inline)) {
+#pragma unroll
+      for (int x = 0; x < Q; ++x) {
+        k4[x] = *reinterpret_cast<const float4*>(&ks[buf][j][x * 4 * DS_PARTS + part * 4]);
+        q4[x] = *reinterpret_cast<const float4*>(&qs[buf][j][x * 4 * DS_PARTS + part * 4]);
+        g4[x] = *reinterpret_cast<const float4*>(&gs[buf][j][x * 4 * DS_PARTS + part * 4]);
+      }
+      v1 = vs[buf][j][col_in];
+      b1 = bs[buf][j];
+      kq1 = kqs[buf][j];
+    };
+    read(0, kk, qq, gg, vv, bb, kqv);
     for (int j = 0; j < batch; ++j) {
+      read(min(j + 1, batch - 1), nk, nq, ng, nv, nb, nkq);
       // One pass decays the rows and forms what the key and the query read of the decayed state (four
       // running sums each, so that the additions do not wait for one another); the token's own write
       // reaches the read-out through k . q: o = (gS)^T q + w (k . q).
       float rk[4] = {0.f, 0.f, 0.f, 0.f}, rq[4] = {0.f, 0.f, 0.f, 0.f};
 #pragma unroll
-      for (int i = 0; i < NR; i += 4) {
-        const float4 kk = *reinterpret_cast<const float4*>(&ks[j][part * NR + i]);
-        const float4 qq = *reinterpret_cast<const float4*>(&qs[j][part * NR + i]);
-        const float4 gg = *reinterpret_cast<const float4*>(&gs[j][part * NR + i]);
-        s[i] *= gg.x; s[i + 1] *= gg.y; s[i + 2] *= gg.z; s[i + 3] *= gg.w;
-        rk[0] = fmaf(s[i], kk.x, rk[0]); rk[1] = fmaf(s[i + 1], kk.y, rk[1]);
-        rk[2] = fmaf(s[i + 2], kk.z, rk[2]); rk[3] = fmaf(s[i + 3], kk.w, rk[3]);
-        rq[0] = fmaf(s[i], qq.x, rq[0]); rq[1] = fmaf(s[i + 1], qq.y, rq[1]);
-        rq[2] = fmaf(s[i + 2], qq.z, rq[2]); rq[3] = fmaf(s[i + 3], qq.w, rq[3]);
+      for (int x = 0; x < Q; ++x) {
+        const int i = 4 * x;
+        s[i] *= gg[x].x; s[i + 1] *= gg[x].y; s[i + 2] *= gg[x].z; s[i + 3] *= gg[x].w;
+        rk[0] = fmaf(s[i], kk[x].x, rk[0]); rk[1] = fmaf(s[i + 1], kk[x].y, rk[1]);
+        rk[2] = fmaf(s[i + 2], kk[x].z, rk[2]); rk[3] = fmaf(s[i + 3], kk[x].w, rk[3]);
+        rq[0] = fmaf(s[i], qq[x].x, rq[0]); rq[1] = fmaf(s[i + 1], qq[x].y, rq[1]);
+        rq[2] = fmaf(s[i + 2], qq[x].z, rq[2]); rq[3] = fmaf(s[i + 3], qq[x].w, rq[3]);
       }
       float read_k = (rk[0] + rk[1]) + (rk[2] + rk[3]), read_q = (rq[0] + rq[1]) + (rq[2] + rq[3]);
-      // Over the eight lanes of the column.
+      // Over the lanes of the column.
       read_k += lanes_moved<0xB1, 0xF>(0.f, read_k);
       read_q += lanes_moved<0xB1, 0xF>(0.f, read_q);
       read_k += lanes_moved<0x4E, 0xF>(0.f, read_k);
       read_q += lanes_moved<0x4E, 0xF>(0.f, read_q);
       read_k += lanes_moved<0x141, 0xF>(0.f, read_k);
       read_q += lanes_moved<0x141, 0xF>(0.f, read_q);
-      const float write = bs[j] * (vs[j][col_in] - read_k);
-#pragma unroll
-      for (int i = 0; i < NR; i += 4) {
-        const float4 kk = *reinterpret_cast<const float4*>(&ks[j][part * NR + i]);
-        s[i] = fmaf(kk.x, write, s[i]); s[i + 1] = fmaf(kk.y, write, s[i + 1]);
-        s[i + 2] = fmaf(kk.z, write, s[i + 2]); s[i + 3] = fmaf(kk.w, write, s[i + 3]);
+      if (DS_PARTS == 16) {  // the two halves of a row of lanes
+        read_k += lanes_moved<0x140, 0xF>(0.f, read_k);
+        read_q += lanes_moved<0x140, 0xF>(0.f, read_q);
       }
-      if (part == 0 && live) o[((size_t)(row0 + base + j) * heads + h) * vdim + c] = fmaf(write, kqs[j], read_q);
+      const float write = bb * (vv - read_k);
+#pragma unroll
+      for (int x = 0; x < Q; ++x) {
+        const int i = 4 * x;
+        s[i] = fmaf(kk[x].x, write, s[i]); s[i + 1] = fmaf(kk[x].y, write, s[i + 1]);
+        s[i + 2] = fmaf(kk[x].z, write, s[i + 2]); s[i + 3] = fmaf(kk[x].w, write, s[i + 3]);
+      }
+      if (part == 0 && live) *o_at = fmaf(write, kqv, read_q);
+      o_at += o_step;
+#pragma unroll
+      for (int x = 0; x < Q; ++x) {
+        kk[x] = nk[x];
+        qq[x] = nq[x];
+        gg[x] = ng[x];
+      }
+      vv = nv;
+      bb = nb;
+      kqv = nkq;
     }
   }
 #pragma unroll
   for (int i = 0; i < NR; ++i) {
-    const int d = part * NR + i;
+    const int d = row_of(i);
     if (live && d < dim) held[(size_t)d * vdim + c] = s[i];
   }
 }
@@ -222,19 +302,28 @@ extern "C" int ts_delta_prepare(float* qn, float* kn, float* kq, float* decay, f
 
 extern "C" int ts_delta_scan(float* o, float* state, const float* qn, const float* kn, const float* kq, const float* decay, const float* beta,
                              const float* u, const int* state_slots, const int* query_start_loc, int first_seq, int num_seqs,
-                             int heads, int kv_heads, int dim, int vdim, hipStream_t stream) {
+                             int heads, int kv_heads, int dim, int vdim, int spread, hipStream_t stream) {
   if (num_seqs == 0) return TS_OK;
   if (!o || !state || !qn || !kn || !kq || !decay || !beta || !u || !state_slots || !query_start_loc) return TS_ERR_ARG;
   if (heads < 1 || kv_heads < 1 || heads % kv_heads != 0 || heads > 65535 || dim < 1 || dim > 256 || vdim < 1) return TS_ERR_SHAPE;
-  const dim3 grid(num_seqs, heads, (vdim + DS_COLS - 1) / DS_COLS), block(DS_PARTS * DS_COLS);
-  if (grid.z > 65535) return TS_ERR_SHAPE;
-#define DS_GO(NR)                                                                                                     \
-  hipLaunchKernelGGL((delta_scan_kernel<NR>), grid, block, 0, stream, o, state, qn, kn, kq, decay, beta, u, state_slots,  \
-                     query_start_loc, first_seq, heads, kv_heads, dim, vdim)
-  if (dim <= 32) DS_GO(4);
-  else if (dim <= 64) DS_GO(8);
-  else if (dim <= 128) DS_GO(16);
-  else DS_GO(32);
+  // `spread` (prompt portions): the state spread thinly; else whole cache lines of the state a workgroup.
+#define DS_GO(NR, BATCH, PARTS, COLS)                                                                                 \
+  do {                                                                                                                \
+    const dim3 grid(num_seqs, heads, (vdim + COLS - 1) / COLS), block(PARTS * COLS);                                  \
+    if (grid.z > 65535) return TS_ERR_SHAPE;                                                                          \
+    hipLaunchKernelGGL((delta_scan_kernel<NR, BATCH, PARTS, COLS>), grid, block, 0, stream, o, state, qn, kn, kq,     \
+                       decay, beta, u, state_slots, query_start_loc, first_seq, heads, kv_heads, dim, vdim);          \
+  } while (0)
+  if (spread) {
+    if (dim <= 64) DS_GO(4, 16, 16, 8);
+    else if (dim <= 128) DS_GO(8, 16, 16, 8);
+    else DS_GO(16, 8, 16, 8);
+  } else {
+    if (dim <= 32) DS_GO(4, 16, 8, 32);
+    else if (dim <= 64) DS_GO(8, 16, 8, 32);
+    else if (dim <= 128) DS_GO(16, 16, 8, 32);
+    else DS_GO(32, 8, 8, 32);
+  }
 #undef DS_GO
   return ts_launch_status();
 }

@@ -100,7 +100,7 @@ _SIGNATURES: dict[str, dict[str, list]] = {
         "ts_delta_prepare": [c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_int, c_long, c_int, c_int,
                              c_int, c_int, c_void_p, c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_int, c_int, c_void_p],
         "ts_delta_scan": [c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_int,
-                          c_int, c_int, c_int, c_int, c_int, c_void_p],
+                          c_int, c_int, c_int, c_int, c_int, c_int, c_void_p],
         "ts_delta_finish": [c_void_p, c_void_p, c_void_p, c_int, c_int, c_long, c_int, c_int, c_int, c_void_p, c_void_p,
                             c_float, c_int, c_int, c_int, c_int, c_void_p],
         "ts_stream_fold": [c_void_p, c_void_p, c_int, c_int, c_long, c_long, c_int, c_int, c_void_p],
@@ -1022,7 +1022,8 @@ class Ops:
     def delta_rule(self, u: torch.Tensor, proj: torch.Tensor, *, beta_at: int, decay_at: int, gate_at: int, a2: torch.Tensor,
                    dt_bias: torch.Tensor, a_log: torch.Tensor, g2: torch.Tensor, gain: torch.Tensor, eps: float,
                    state: torch.Tensor, state_slots: torch.Tensor, query_start_loc: torch.Tensor, tokens: int, num_seqs: int,
-                   heads: int, kv_heads: int, head_dim: int, value_dim: int, dtype: torch.dtype) -> torch.Tensor:
+                   heads: int, kv_heads: int, head_dim: int, value_dim: int, dtype: torch.dtype,
+                   num_long_seqs: int = 0) -> torch.Tensor:
         """The gated delta rule over a step: per head and request a 32-bit state ``S [D, Dv]`` (``state [slots, H,
         D, Dv]``) that every token decays, corrects and reads: ``S <- diag(g) S; w = beta (v - S^T k); S <- S + k
         w^T; o = S^T q``.  ``u [T, 2 G D + H Dv]`` (32-bit) holds the step's convolved ``q | k | v``; ``q`` and ``k``
@@ -1030,7 +1031,9 @@ class Ops:
         dt_bias))`` with ``low`` the ``a2.shape[1]`` columns of ``proj`` from ``decay_at`` on, ``beta`` the sigmoid of
         the ``H`` columns from ``beta_at`` on.  Every head's ``o`` is divided by its root mean square, multiplied
         by ``gain [Dv]`` and by ``sigmoid(g2 . low')``, ``low'`` the ``g2.shape[1]`` columns from ``gate_at`` on.
-        Returns ``[T, H Dv]`` of ``dtype``."""
+        The first ``num_long_seqs`` requests (those that bring several tokens) are walked with the state spread
+        thinly over many workgroups, the others with whole cache lines of the state a workgroup.  Returns ``[T, H
+        Dv]`` of ``dtype``."""
         _gpu(u, proj, a2, dt_bias, a_log, g2, gain, state, state_slots, query_start_loc)
         _i32(state_slots, "state_slots")
         _i32(query_start_loc, "query_start_loc")
@@ -1060,9 +1063,10 @@ class Ops:
         _check(self.core.ts_delta_prepare(_ptr(qn), _ptr(kn), _ptr(kq), _ptr(decay), _ptr(beta), _ptr(u), _ptr(proj), is_f32, splits, stride,
                                           width, beta_at, decay_at, a2.shape[1], _ptr(a2), _ptr(dt_bias), _ptr(a_log), tokens,
                                           heads, kv_heads, head_dim, value_dim, code, self.stream()), "ts_delta_prepare")
-        _check(self.core.ts_delta_scan(_ptr(o), _ptr(state), _ptr(qn), _ptr(kn), _ptr(kq), _ptr(decay), _ptr(beta), _ptr(u), _ptr(state_slots),
-                                       _ptr(query_start_loc), 0, num_seqs, heads, kv_heads, head_dim, value_dim, self.stream()),
-               "ts_delta_scan")
+        for first, count, spread in ((0, num_long_seqs, 1), (num_long_seqs, num_seqs - num_long_seqs, 0)):
+            _check(self.core.ts_delta_scan(_ptr(o), _ptr(state), _ptr(qn), _ptr(kn), _ptr(kq), _ptr(decay), _ptr(beta), _ptr(u),
+                                           _ptr(state_slots), _ptr(query_start_loc), first, count, heads, kv_heads, head_dim,
+                                           value_dim, spread, self.stream()), "ts_delta_scan")
         y = self.rows_buffer(tokens, values, dtype, device)
         _check(self.core.ts_delta_finish(_ptr(y), _ptr(o), _ptr(proj), is_f32, splits, stride, width, gate_at, g2.shape[1], _ptr(g2),
                                          _ptr(gain), float(eps), tokens, heads, value_dim, code, self.stream()), "ts_delta_finish")

@@ -129,5 +129,6 @@ class GatedDeltaRule(Mixer):
                            dt_bias=self.dt, a_log=self.a_log, g2=self.g2, gain=self.gain, eps=self.norm_eps,
                            state=memory.state, state_slots=ctx.state_slots, query_start_loc=ctx.query_start_loc,
                            tokens=ctx.num_tokens, num_seqs=ctx.num_seqs, heads=self.num_heads, kv_heads=self.num_kv_heads,
-                           head_dim=self.head_dim, value_dim=self.value_dim, dtype=dtype)
+                           head_dim=self.head_dim, value_dim=self.value_dim, dtype=dtype,
+                           num_long_seqs=0 if ctx.recorded else ctx.num_prefill_seqs)
         return ops.linear(y, self.o_weight, for_residual=True)

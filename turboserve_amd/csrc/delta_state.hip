@@ -110,6 +110,8 @@ delta_scan_kernel(float* __restrict__ o, float* __restrict__ state, const float*
   __shared__ __attribute__((aligned(16))) float gs[2][BATCH][ROWS];
   __shared__ float vs[2][BATCH][DS_COLS];
   __shared__ float bs[2][BATCH], kqs[2][BATCH];
+  __shared__ __attribute__((aligned(16))) float read_q_of[BATCH][THREADS];  // per token and lane: what the query reads of the lane's rows
+  __shared__ float write_of[BATCH][DS_COLS];
   const int seq = first_seq + blockIdx.x, h = blockIdx.y;
   const int g = h / (heads / kv_heads);
   const int tid = threadIdx.x;
@@ -186,10 +188,13 @@ delta_scan_kernel(float* __restrict__ o, float* __restrict__ state, const float*
     // In flight while this batch is walked; asked for unconditionally (behind the last batch: the last
     // token again, which nobody stages), so that no wait for it is placed inside the walk.
     fetch(min(base + BATCH, count - 1));
-    // A token's vectors are read from LDS while the token before it is walked.
-    float4 kk[Q], qq[Q], gg[Q], nk[Q], nq[Q], ng[Q];
-    float vv, bb, kqv, nv, nb, nkq;
-    auto read = [&](int j, float4* k4, float4* q4, float4* g4, float& v1, float& b1, float& kq1) __attribute__((always_inline)) {
+    // A token's vectors are read from LDS while the token before it is walked (two sets of registers in
+    // turn).  What the query reads is left in LDS lane by lane and summed over a column's lanes behind the
+    // batch, all tokens side by side: only the key's read-out, which the state's update waits for, crosses
+    // lanes inside the walk.
+    float4 ka[Q], qa[Q], ga[Q], kb[Q], qb[Q], gb[Q];
+    float va, ba, vb, bb;
+    auto read = [&](int j, float4* k4, float4* q4, float4* g4, float& v1, float& b1) __attribute__((always_inline)) {
 #pragma unroll
       for (int x = 0; x < Q; ++x) {
         k4[x] = *reinterpret_cast<const float4*>(&ks[buf][j][x * 4 * DS_PARTS + part * 4]);
@@ -198,11 +203,8 @@ delta_scan_kernel(float* __restrict__ o, float* __restrict__ state, const float*
       }
       v1 = vs[buf][j][col_in];
       b1 = bs[buf][j];
-      kq1 = kqs[buf][j];
     };
-    read(0, kk, qq, gg, vv, bb, kqv);
-    for (int j = 0; j < batch; ++j) {
-      read(min(j + 1, batch - 1), nk, nq, ng, nv, nb, nkq);
+    auto token = [&](int j, const float4* kk, const float4* qq, const float4* gg, float vv, float beta_j) __attribute__((always_inline)) {
       // One pass decays the rows and forms what the key and the query read of the decayed state (four
       // running sums each, so that the additions do not wait for one another); the token's own write
       // reaches the read-out through k . q: o = (gS)^T q + w (k . q).
@@ -216,37 +218,43 @@ delta_scan_kernel(float* __restrict__ o, float* __restrict__ state, const float*
         rq[0] = fmaf(s[i], qq[x].x, rq[0]); rq[1] = fmaf(s[i + 1], qq[x].y, rq[1]);
         rq[2] = fmaf(s[i + 2], qq[x].z, rq[2]); rq[3] = fmaf(s[i + 3], qq[x].w, rq[3]);
       }
-      float read_k = (rk[0] + rk[1]) + (rk[2] + rk[3]), read_q = (rq[0] + rq[1]) + (rq[2] + rq[3]);
+      float read_k = (rk[0] + rk[1]) + (rk[2] + rk[3]);
+      read_q_of[j][tid] = (rq[0] + rq[1]) + (rq[2] + rq[3]);
       // Over the lanes of the column.
       read_k += lanes_moved<0xB1, 0xF>(0.f, read_k);
-      read_q += lanes_moved<0xB1, 0xF>(0.f, read_q);
       read_k += lanes_moved<0x4E, 0xF>(0.f, read_k);
-      read_q += lanes_moved<0x4E, 0xF>(0.f, read_q);
       read_k += lanes_moved<0x141, 0xF>(0.f, read_k);
-      read_q += lanes_moved<0x141, 0xF>(0.f, read_q);
-      if (DS_PARTS == 16) {  // the two halves of a row of lanes
-        read_k += lanes_moved<0x140, 0xF>(0.f, read_k);
-        read_q += lanes_moved<0x140, 0xF>(0.f, read_q);
-      }
-      const float write = bb * (vv - read_k);
+      if (DS_PARTS == 16) read_k += lanes_moved<0x140, 0xF>(0.f, read_k);  // the two halves of a row of lanes
+      const float write = beta_j * (vv - read_k);
+      write_of[j][col_in] = write;  // (every lane of the column writes the same number)
 #pragma unroll
       for (int x = 0; x < Q; ++x) {
         const int i = 4 * x;
         s[i] = fmaf(kk[x].x, write, s[i]); s[i + 1] = fmaf(kk[x].y, write, s[i + 1]);
         s[i + 2] = fmaf(kk[x].z, write, s[i + 2]); s[i + 3] = fmaf(kk[x].w, write, s[i + 3]);
       }
-      if (part == 0 && live) *o_at = fmaf(write, kqv, read_q);
-      o_at += o_step;
-#pragma unroll
-      for (int x = 0; x < Q; ++x) {
-        kk[x] = nk[x];
-        qq[x] = nq[x];
-        gg[x] = ng[x];
+    };
+    read(0, ka, qa, ga, va, ba);
+    for (int j = 0; j < batch; j += 2) {
+      read(min(j + 1, batch - 1), kb, qb, gb, vb, bb);
+      token(j, ka, qa, ga, va, ba);
+      if (j + 1 < batch) {
+        read(min(j + 2, batch - 1), ka, qa, ga, va, ba);
+        token(j + 1, kb, qb, gb, vb, bb);
       }
-      vv = nv;
-      bb = nb;
-      kqv = nkq;
     }
+    // The batch's outputs: lane `part` of a column sums what the column's lanes left for the tokens part,
+    // part + DS_PARTS, ..  (A column's lanes are one wavefront's, whose LDS accesses keep their order.)
+    for (int j = part; j < batch; j += DS_PARTS) {
+      float sum = 0.f;
+#pragma unroll
+      for (int x = 0; x < DS_PARTS / 4; ++x) {
+        const float4 piece = *reinterpret_cast<const float4*>(&read_q_of[j][col_in * DS_PARTS + 4 * x]);
+        sum += (piece.x + piece.y) + (piece.z + piece.w);
+      }
+      if (live) o_at[(size_t)j * o_step] = fmaf(write_of[j][col_in], kqs[buf][j], sum);
+    }
+    o_at += (size_t)batch * o_step;
   }
 #pragma unroll
   for (int i = 0; i < NR; ++i) {
@@ -319,9 +327,9 @@ extern "C" int ts_delta_scan(float* o, float* state, const float* qn, const floa
     else if (dim <= 128) DS_GO(8, 16, 16, 8);
     else DS_GO(16, 8, 16, 8);
   } else {
-    if (dim <= 32) DS_GO(4, 16, 8, 32);
-    else if (dim <= 64) DS_GO(8, 16, 8, 32);
-    else if (dim <= 128) DS_GO(16, 16, 8, 32);
+    if (dim <= 32) DS_GO(4, 8, 8, 32);
+    else if (dim <= 64) DS_GO(8, 8, 8, 32);
+    else if (dim <= 128) DS_GO(16, 8, 8, 32);
     else DS_GO(32, 8, 8, 32);
   }
 #undef DS_GO

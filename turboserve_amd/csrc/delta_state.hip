@@ -11,6 +11,9 @@
 //                     from and to the request's slot;
 //   ts_delta_finish   per (token, head): o divided by its root mean square, times a gain [Dv] shared by
 //                     the heads, times sigmoid(g2 . low'), rounded once to the run's type.
+// Of the two low-rank matrices a2 [H D, R] and g2 [H Dv, R'] a lane walks its channel's row; over a prompt a
+// wavefront of the launches around the walk takes eight tokens, so that it reads its rows once for all eight (in a
+// step of few tokens: one token each).
 // `u` [T, 2 G D + H Dv] (32-bit) holds the convolved q | k | v; `proj` is the fused projection [T, width]
 // of the run's type, or `splits` 32-bit partial sums, of which the columns named by *_at are read.
 #include "common.hpp"
@@ -32,19 +35,25 @@ __device__ __forceinline__ float ds_input(const P* p, int splits, size_t stride)
   return s;
 }
 
-// Block (t, item): item < G makes key head `item`'s unit q and k; item >= G the decays and beta of head
-// item - G.
-template <typename T, typename P>
-__global__ void __launch_bounds__(64)
+// A workgroup of four wavefronts, each with an item of its own.  The first `qk_blocks` workgroups make unit q
+// and k: item = (token, key head).  The others make decays and beta: item = (tile of DS_TOKENS tokens, head).
+// A lane walks its channel's row of the low-rank matrix once (neighbouring elements: wide loads) for all the
+// tile's tokens, whose low-rank inputs lie side by side in the wavefront's own stretch of LDS.
+#define DS_ITEMS 4
+template <typename T, typename P, int DS_TOKENS>
+__global__ void __launch_bounds__(64 * DS_ITEMS)
 delta_prepare_kernel(float* __restrict__ qn, float* __restrict__ kn, float* __restrict__ kq, float* __restrict__ decay,
                      float* __restrict__ beta, const float* __restrict__ u, const P* __restrict__ proj, int splits, size_t split_stride, int width,
                      int beta_at, int low_at, int low, const T* __restrict__ a2, const T* __restrict__ dt_bias,
-                     const float* __restrict__ a_log, int heads, int kv_heads, int dim, int vdim) {
-  __shared__ float lows[DS_MAX_LOW];
-  const int t = blockIdx.x, item = blockIdx.y, lane = threadIdx.x;
+                     const float* __restrict__ a_log, int tokens, int heads, int kv_heads, int dim, int vdim, int qk_blocks) {
+  __shared__ __attribute__((aligned(16))) float lows_of[DS_ITEMS][DS_MAX_LOW][DS_TOKENS];  // the tokens of a tile side by side
+  const int wave = threadIdx.x / TS_WAVE, lane = threadIdx.x % TS_WAVE;
   const size_t u_width = (size_t)2 * kv_heads * dim + (size_t)heads * vdim;
-  if (item < kv_heads) {
-    const float* q = u + (size_t)t * u_width + (size_t)item * dim;
+  if ((int)blockIdx.x < qk_blocks) {
+    const long item = (long)blockIdx.x * DS_ITEMS + wave;
+    if (item >= (long)tokens * kv_heads) return;
+    const int t = (int)(item / kv_heads), g = (int)(item % kv_heads);
+    const float* q = u + (size_t)t * u_width + (size_t)g * dim;
     const float* k = q + (size_t)kv_heads * dim;
     float qq = 0.f, kk = 0.f;
     for (int d = lane; d < dim; d += TS_WAVE) {
@@ -54,7 +63,7 @@ delta_prepare_kernel(float* __restrict__ qn, float* __restrict__ kn, float* __re
     qq = wave_sum(qq);
     kk = wave_sum(kk);
     const float q_by = rsqrtf(qq + 1e-6f) * rsqrtf((float)dim), k_by = rsqrtf(kk + 1e-6f);
-    const size_t at = ((size_t)t * kv_heads + item) * dim;
+    const size_t at = ((size_t)t * kv_heads + g) * dim;
     float both = 0.f;
     for (int d = lane; d < dim; d += TS_WAVE) {
       const float qd = q[d] * q_by, kd = k[d] * k_by;
@@ -63,22 +72,44 @@ delta_prepare_kernel(float* __restrict__ qn, float* __restrict__ kn, float* __re
       both = fmaf(kd, qd, both);
     }
     both = wave_sum(both);
-    if (lane == 0) kq[(size_t)t * kv_heads + item] = both;
+    if (lane == 0) kq[(size_t)t * kv_heads + g] = both;
     return;
   }
-  const int h = item - kv_heads;
-  const P* row = proj + (size_t)t * width;
-  for (int r = lane; r < low; r += TS_WAVE) lows[r] = ds_input(row + low_at + r, splits, split_stride);
+  // (Every wavefront of such a workgroup reaches the barrier; one without an item does nothing around it.)
+  const int tiles = (tokens + DS_TOKENS - 1) / DS_TOKENS;
+  const long item = (long)((int)blockIdx.x - qk_blocks) * DS_ITEMS + wave;
+  const bool mine = item < (long)tiles * heads;
+  const int h = mine ? (int)(item % heads) : 0;
+  const int t0 = mine ? (int)(item / heads) * DS_TOKENS : 0;
+  const int count = mine ? min(DS_TOKENS, tokens - t0) : 0;
+  float (*lows)[DS_TOKENS] = lows_of[wave];
+  for (int i = lane; i < DS_TOKENS * low; i += TS_WAVE) {
+    const int tt = i / low, r = i % low;
+    lows[r][tt] = tt < count ? ds_input(proj + (size_t)(t0 + tt) * width + low_at + r, splits, split_stride) : 0.f;
+  }
   __syncthreads();
-  if (lane == 0) beta[(size_t)t * heads + h] = 1.f / (1.f + expf(-ds_input(row + beta_at + h, splits, split_stride)));
+  if (!mine) return;
+  if (lane < count)
+    beta[(size_t)(t0 + lane) * heads + h] = 1.f / (1.f + expf(-ds_input(proj + (size_t)(t0 + lane) * width + beta_at + h, splits, split_stride)));
   const float rate = expf(a_log[h]);
   for (int d = lane; d < dim; d += TS_WAVE) {
     const size_t channel = (size_t)h * dim + d;
     const T* w = a2 + channel * low;
-    float z = to_float(dt_bias[channel]);
-    for (int r = 0; r < low; ++r) z = fmaf(to_float(w[r]), lows[r], z);
-    const float step = z > 20.f ? z : log1pf(expf(z));
-    decay[((size_t)t * heads + h) * dim + d] = expf(-rate * step);
+    float z[DS_TOKENS];
+#pragma unroll
+    for (int tt = 0; tt < DS_TOKENS; ++tt) z[tt] = to_float(dt_bias[channel]);
+    for (int r = 0; r < low; ++r) {
+      const float wr = to_float(w[r]);
+#pragma unroll
+      for (int tt = 0; tt < DS_TOKENS; ++tt) z[tt] = fmaf(wr, lows[r][tt], z[tt]);
+    }
+#pragma unroll
+    for (int tt = 0; tt < DS_TOKENS; ++tt) {
+      if (tt < count) {
+        const float step = z[tt] > 20.f ? z[tt] : log1pf(expf(z[tt]));
+        decay[((size_t)(t0 + tt) * heads + h) * dim + d] = expf(-rate * step);
+      }
+    }
   }
 }
 
@@ -263,26 +294,54 @@ delta_scan_kernel(float* __restrict__ o, float* __restrict__ state, const float*
   }
 }
 
-template <typename T, typename P>
-__global__ void __launch_bounds__(64)
+// Four wavefronts a workgroup, each with an item (tile of DS_TOKENS tokens, head) of its own.
+template <typename T, typename P, int DS_TOKENS>
+__global__ void __launch_bounds__(64 * DS_ITEMS)
 delta_finish_kernel(T* __restrict__ y, const float* __restrict__ o, const P* __restrict__ proj, int splits, size_t split_stride,
-                    int width, int low_at, int low, const T* __restrict__ g2, const T* __restrict__ gain, float eps, int heads,
-                    int vdim) {
-  __shared__ float lows[DS_MAX_LOW];
-  const int t = blockIdx.x, h = blockIdx.y, lane = threadIdx.x;
-  const P* row = proj + (size_t)t * width;
-  for (int r = lane; r < low; r += TS_WAVE) lows[r] = ds_input(row + low_at + r, splits, split_stride);
+                    int width, int low_at, int low, const T* __restrict__ g2, const T* __restrict__ gain, float eps, int tokens,
+                    int heads, int vdim) {
+  __shared__ __attribute__((aligned(16))) float lows_of[DS_ITEMS][DS_MAX_LOW][DS_TOKENS];
+  const int wave = threadIdx.x / TS_WAVE, lane = threadIdx.x % TS_WAVE;
+  const int tiles = (tokens + DS_TOKENS - 1) / DS_TOKENS;
+  const long item = (long)blockIdx.x * DS_ITEMS + wave;
+  const bool mine = item < (long)tiles * heads;
+  const int h = mine ? (int)(item % heads) : 0;
+  const int t0 = mine ? (int)(item / heads) * DS_TOKENS : 0;
+  const int count = mine ? min(DS_TOKENS, tokens - t0) : 0;
+  float (*lows)[DS_TOKENS] = lows_of[wave];
+  for (int i = lane; i < DS_TOKENS * low; i += TS_WAVE) {
+    const int tt = i / low, r = i % low;
+    lows[r][tt] = tt < count ? ds_input(proj + (size_t)(t0 + tt) * width + low_at + r, splits, split_stride) : 0.f;
+  }
   __syncthreads();
-  const float* mine = o + ((size_t)t * heads + h) * vdim;
-  float ss = 0.f;
-  for (int c = lane; c < vdim; c += TS_WAVE) ss = fmaf(mine[c], mine[c], ss);
-  ss = wave_sum(ss);
-  const float by = rsqrtf(ss / (float)vdim + eps);
+  if (!mine) return;
+  float by[DS_TOKENS];
+#pragma unroll
+  for (int tt = 0; tt < DS_TOKENS; ++tt) {
+    const float* mine_o = o + ((size_t)(t0 + min(tt, count - 1)) * heads + h) * vdim;
+    float ss = 0.f;
+    for (int c = lane; c < vdim; c += TS_WAVE) ss = fmaf(mine_o[c], mine_o[c], ss);
+    ss = wave_sum(ss);
+    by[tt] = rsqrtf(ss / (float)vdim + eps);
+  }
   for (int c = lane; c < vdim; c += TS_WAVE) {
     const T* w = g2 + ((size_t)h * vdim + c) * low;
-    float z = 0.f;
-    for (int r = 0; r < low; ++r) z = fmaf(to_float(w[r]), lows[r], z);
-    y[((size_t)t * heads + h) * vdim + c] = from_float<T>(mine[c] * by * to_float(gain[c]) / (1.f + expf(-z)));
+    float z[DS_TOKENS];
+#pragma unroll
+    for (int tt = 0; tt < DS_TOKENS; ++tt) z[tt] = 0.f;
+    for (int r = 0; r < low; ++r) {
+      const float wr = to_float(w[r]);
+#pragma unroll
+      for (int tt = 0; tt < DS_TOKENS; ++tt) z[tt] = fmaf(wr, lows[r][tt], z[tt]);
+    }
+    const float g = to_float(gain[c]);
+#pragma unroll
+    for (int tt = 0; tt < DS_TOKENS; ++tt) {
+      if (tt < count) {
+        const size_t at = ((size_t)(t0 + tt) * heads + h) * vdim + c;
+        y[at] = from_float<T>(o[at] * by[tt] * g / (1.f + expf(-z[tt])));
+      }
+    }
   }
 }
 
@@ -295,11 +354,19 @@ extern "C" int ts_delta_prepare(float* qn, float* kn, float* kq, float* decay, f
   if (heads < 1 || kv_heads < 1 || heads % kv_heads != 0 || heads + kv_heads > 65535 || dim < 1 || vdim < 1 || low < 1 ||
       low > DS_MAX_LOW || splits < 1 || beta_at < 0 || beta_at + heads > width || low_at < 0 || low_at + low > width)
     return TS_ERR_SHAPE;
-  const dim3 grid(tokens, kv_heads + heads), block(64);
+  // Eight tokens a tile over a prompt; one in a step of few tokens, whose workgroups are few anyway.
+  const int per = tokens >= 64 ? 8 : 1;
+  const int qk_blocks = (int)(((long)tokens * kv_heads + DS_ITEMS - 1) / DS_ITEMS);
+  const long decay_items = (long)((tokens + per - 1) / per) * heads;
+  const dim3 grid((unsigned)(qk_blocks + (decay_items + DS_ITEMS - 1) / DS_ITEMS)), block(64 * DS_ITEMS);
+#define DS_ARGS(T, P)                                                                                                    \
+  grid, block, 0, stream, qn, kn, kq, decay, beta, u, (const P*)proj, splits, (size_t)split_stride, width, beta_at, low_at, \
+      low, (const T*)a2, (const T*)dt_bias, a_log, tokens, heads, kv_heads, dim, vdim, qk_blocks
 #define DS_GO(T, P)                                                                                                      \
-  hipLaunchKernelGGL((delta_prepare_kernel<T, P>), grid, block, 0, stream, qn, kn, kq, decay, beta, u, (const P*)proj, splits, \
-                     (size_t)split_stride, width, beta_at, low_at, low, (const T*)a2, (const T*)dt_bias, a_log, heads,    \
-                     kv_heads, dim, vdim)
+  if (per == 8)                                                                                                          \
+    hipLaunchKernelGGL((delta_prepare_kernel<T, P, 8>), DS_ARGS(T, P));                                                  \
+  else                                                                                                                   \
+    hipLaunchKernelGGL((delta_prepare_kernel<T, P, 1>), DS_ARGS(T, P))
   if (dtype == TS_F32) DS_GO(float, float);
   else if (dtype == TS_BF16 && in_f32) DS_GO(bf16_t, float);
   else if (dtype == TS_BF16) DS_GO(bf16_t, bf16_t);
@@ -343,10 +410,16 @@ extern "C" int ts_delta_finish(void* y, const float* o, const void* proj, int in
   if (!y || !o || !proj || !g2 || !gain) return TS_ERR_ARG;
   if (heads < 1 || heads > 65535 || vdim < 1 || low < 1 || low > DS_MAX_LOW || splits < 1 || low_at < 0 || low_at + low > width)
     return TS_ERR_SHAPE;
-  const dim3 grid(tokens, heads), block(64);
+  const int per = tokens >= 64 ? 8 : 1;
+  const long items = (long)((tokens + per - 1) / per) * heads;
+  const dim3 grid((unsigned)((items + DS_ITEMS - 1) / DS_ITEMS)), block(64 * DS_ITEMS);
 #define DS_GO(T, P)                                                                                                   \
-  hipLaunchKernelGGL((delta_finish_kernel<T, P>), grid, block, 0, stream, (T*)y, o, (const P*)proj, splits,            \
-                     (size_t)split_stride, width, low_at, low, (const T*)g2, (const T*)gain, eps, heads, vdim)
+  if (per == 8)                                                                                                       \
+    hipLaunchKernelGGL((delta_finish_kernel<T, P, 8>), grid, block, 0, stream, (T*)y, o, (const P*)proj, splits,       \
+                       (size_t)split_stride, width, low_at, low, (const T*)g2, (const T*)gain, eps, tokens, heads, vdim); \
+  else                                                                                                                \
+    hipLaunchKernelGGL((delta_finish_kernel<T, P, 1>), grid, block, 0, stream, (T*)y, o, (const P*)proj, splits,       \
+                       (size_t)split_stride, width, low_at, low, (const T*)g2, (const T*)gain, eps, tokens, heads, vdim)
   if (dtype == TS_F32) DS_GO(float, float);
   else if (dtype == TS_BF16 && in_f32) DS_GO(bf16_t, float);
   else if (dtype == TS_BF16) DS_GO(bf16_t, bf16_t);

@@ -94,7 +94,7 @@ _SIGNATURES: dict[str, dict[str, list]] = {
                              c_int, c_int, c_void_p, c_int, c_long, c_void_p],
         "ts_tanh_cap": [c_void_p, c_long, c_float, c_void_p],
         "ts_short_conv": [c_void_p, c_int, c_void_p, c_int, c_int, c_long, c_int, c_int, c_int, c_void_p, c_int, c_void_p,
-                          c_void_p, c_void_p, c_void_p, c_int, c_int, c_int, c_void_p],
+                          c_void_p, c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_void_p],
         "ts_short_conv_carry": [c_void_p, c_void_p, c_int, c_int, c_long, c_int, c_int, c_int, c_int, c_void_p, c_void_p,
                                 c_int, c_int, c_void_p],
         "ts_delta_prepare": [c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_int, c_long, c_int, c_int,
@@ -1011,9 +1011,13 @@ class Ops:
         out = torch.empty((tokens, channels), dtype=torch.float32, device=proj.device) if wide \
             else self.rows_buffer(tokens, channels, dtype, proj.device)
         code = dtype_code(dtype)
+        # Every request brings one token: the launch that convolves also moves the state on.
+        single = tokens == num_seqs
         _check(self.core.ts_short_conv(_ptr(out), 1 if wide else 0, _ptr(proj), is_f32, splits, stride, width, first_col, channels,
                                        _ptr(taps), k, _ptr(state), _ptr(state_slots), _ptr(token_seq), _ptr(query_start_loc),
-                                       tokens, 1 if silu else 0, code, self.stream()), "ts_short_conv")
+                                       tokens, 1 if silu else 0, 1 if single else 0, code, self.stream()), "ts_short_conv")
+        if single:
+            return out
         _check(self.core.ts_short_conv_carry(_ptr(state), _ptr(proj), is_f32, splits, stride, width, first_col, channels, k,
                                              _ptr(state_slots), _ptr(query_start_loc), num_seqs, code, self.stream()),
                "ts_short_conv_carry")

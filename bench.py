@@ -560,7 +560,7 @@ def legavik_pair(size: str) -> tuple[dict, dict]:
     keyed = {"heads": heads, "kv_heads": kv, "dim": 128, "vdim": 128, "scale": 128 ** -0.5, "mask": {"size": 1024, "keep_first": 64},
              "rot": {"base": 10000.0, "dims": 64, "scaling": {"factor": 8.0, "original": 1024, "fast": 32.0, "slow": 1.0}}}
     order = ["parallel", "attention", "parallel", "parallel", "attention", "parallel"]
-    legavik = {"architecture": "Legavik", "vocab": 32000, "width": width, "norm": {"eps": 1e-6}, "logit_softcap": 30.0,
+    legavik = {"architecture": "Legavik", "vocab": 32000, "width": width, "norm": {"eps": 1e-6}, "logit_softcap": 50.0,
                "layers": [{"type": kind, "mixer": pair if kind == "parallel" else keyed, "mlp": routed} for kind in order]}
     attention = {"heads": heads, "kv_heads": kv, "dim": 128, "vdim": 128, "scale": 128 ** -0.5}
     beside_routed = {"kind": "moe", "expert": {"ff": expert_ff, "limit": 7.0}, "router": {"experts": experts, "top": top}}

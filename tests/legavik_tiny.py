@@ -74,7 +74,7 @@ CONFIG_B = {
     "architecture": "Legavik", "vocab": 97, "width": 52, "norm": {"eps": 1e-6},
     "layers": [
         layer(keyed(1, 1, 12, scale=0.4, window=1, keep=3, rot=4, base=50.0), moe(28, 3, 1, (3, 1))),
-        layer(parallel(left(5, 5, 12, 12, 1, scale=0.5), right(3, 3, 12, 20, 5, 4, 4), 0.6, 0.9), moe(20, 5, 2, (5, 3))),
+        layer(parallel(left(5, 5, 12, 12, 1, scale=0.5), right(3, 3, 12, 20, 5, 4, 4), 0.45, 1.3), moe(20, 5, 2, (5, 3))),
         layer(keyed(2, 2, 6, window=7, rot=6, stretch=(2.0, 16, 4.0, 0.5), base=300.0), None),
         layer(keyed(3, 3, 20, scale=0.3), moe(12, 2, 2)),
         layer(parallel(left(1, 1, 20, 36, 4, temp=(1.0, 1)), right(1, 1, 20, 12, 1, 2, 9), -0.8, 1.0), None),
@@ -85,10 +85,10 @@ PAGE_B = 8
 #: C: heads on the matrix-core path, windows of several pages, kept tokens of more than a page, key
 #: channels beyond 64 on the right, pages of 32.
 CONFIG_C = {
-    "architecture": "Legavik", "vocab": 160, "width": 96, "norm": {"eps": 1e-6}, "logit_softcap": 30.0,
+    "architecture": "Legavik", "vocab": 160, "width": 96, "norm": {"eps": 1e-6}, "logit_softcap": 25.0,
     "layers": [
-        layer(keyed(6, 2, 32, window=70, keep=40, rot=16, stretch=(6.0, 128, 24.0, 2.0), base=200000.0), moe(48, 8, 4, (4, 3))),
-        layer(parallel(left(4, 4, 32, 64, 3, temp=(0.3, 64)), right(4, 2, 96, 32, 4, 8, 8), 0.6, 0.9), moe(64, 8, 2, (2, 1))),
+        layer(keyed(6, 2, 32, window=70, keep=40, rot=16, stretch=(6.0, 128, 24.0, 2.0), base=200000.0), moe(48, 10, 4, (5, 3))),
+        layer(parallel(left(4, 4, 32, 64, 3, temp=(0.25, 48)), right(4, 2, 96, 32, 4, 8, 8), 0.8, 0.55), moe(64, 8, 2, (2, 1))),
         layer(keyed(8, 1, 64, window=33, keep=1, rot=64), None),
         layer(parallel(left(8, 2, 16, 16, 3), right(2, 2, 40, 72, 3, 16, 4), 1.0, 1.0), moe(32, 6, 6)),
     ],

@@ -112,7 +112,7 @@ def test_the_norm_without_statistics_carries_the_residual_sum(ops, dtype, hidden
 
 def test_the_cap_on_the_logits(ops):
     x = torch.linspace(-90, 90, 1001).reshape(7, 143).contiguous()
-    near(ops.tanh_cap(x.clone().to(DEV), 30.0), 30.0 * torch.tanh(x / 30.0), torch.float32)
+    near(ops.tanh_cap(x.clone().to(DEV), 22.0), 22.0 * torch.tanh(x / 22.0), torch.float32)
 
 
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
@@ -234,7 +234,7 @@ def test_the_delta_rule_whole_and_in_pieces(ops, dtype, heads, kv_heads, dim, vd
         assert torch.isnan(state[[0, 2, 4]]).all()
 
 
-@pytest.mark.parametrize("experts,top,groups,keep", [(8, 4, 4, 3), (6, 2, 3, 2), (5, 2, 5, 3), (4, 4, 1, 1), (12, 3, 2, 1)])
+@pytest.mark.parametrize("experts,top,groups,keep", [(10, 4, 5, 3), (6, 2, 3, 2), (5, 2, 5, 3), (4, 4, 1, 1), (12, 3, 2, 1)])
 def test_the_router_marks_a_group_by_its_best_expert(ops, experts, top, groups, keep):
     g = torch.Generator().manual_seed(experts * 10 + top)
     x = torch.randn(50, 24, generator=g)
@@ -274,7 +274,7 @@ def plain_rows(q, k, v, contexts, scale, window, keep):
 
 @pytest.mark.parametrize("heads,kv_heads,dim,vdim,page,window,keep", [
     (4, 2, 16, 16, 16, 20, 5), (3, 1, 24, 8, 8, 1, 3), (6, 2, 32, 32, 32, 70, 40), (8, 1, 64, 128, 16, 33, 1),
-    (2, 2, 128, 128, 16, 136, 20), (4, 4, 64, 64, 8, 64, 64), (2, 1, 8, 8, 8, 9, 0), (1, 1, 40, 24, 16, 300, 7)])
+    (2, 2, 128, 128, 16, 150, 24), (4, 4, 64, 64, 8, 64, 64), (2, 1, 8, 8, 8, 9, 0), (1, 1, 40, 24, 16, 300, 7)])
 def test_a_window_that_keeps_the_first_keys(ops, heads, kv_heads, dim, vdim, page, window, keep):
     """Portions and single tokens in one step, pages scattered and those between the kept keys and the window
     missing: the generic kernel in 32-bit against explicit rows, the tiled kernel in bfloat16 against both."""
@@ -335,11 +335,14 @@ ALONE = {
     "keyed_window_of_one": lt.layer(lt.keyed(3, 3, 8, scale=0.5, window=1, keep=2, rot=2), None),
     "keyed_no_rotation": lt.layer(lt.keyed(2, 1, 12, window=9), None),
     "keyed_matrix_cores": lt.layer(lt.keyed(4, 1, 32, window=40, keep=17, rot=16, stretch=(2.0, 16, 4.0, 1.0), base=5000.0), None),
+    # No kept tokens: keys and values of one size go to the head-size kernels, with and without a window.
+    "keyed_head_size_kernels": lt.layer(lt.keyed(4, 2, 32, window=40, rot=16, base=300.0), None),
+    "keyed_head_size_kernels_no_window": lt.layer(lt.keyed(4, 1, 64, rot=32, stretch=(4.0, 32, 8.0, 1.0)), None),
     "left_only_matters": lt.layer(lt.parallel(lt.left(4, 2, 16, 24, 3, scale=0.4, temp=(0.5, 4)), lt.right(1, 1, 8, 8, 2, 2, 2), 1.0, 1e-3), None),
     "right_only_matters": lt.layer(lt.parallel(lt.left(1, 1, 8, 8, 2), lt.right(4, 2, 16, 12, 4, 5, 3), 1e-3, 1.0), None),
     "pair_one_tap": lt.layer(lt.parallel(lt.left(2, 2, 8, 16, 1, temp=(1.0, 1)), lt.right(2, 2, 8, 8, 1, 3, 3), 0.5, -0.7), None),
-    "pair_matrix_cores": lt.layer(lt.parallel(lt.left(4, 2, 32, 64, 3, temp=(0.3, 16)), lt.right(2, 1, 72, 40, 3, 8, 8), 0.6, 0.9), None),
-    "experts": lt.layer(lt.keyed(1, 1, 8, rot=4), lt.moe(20, 8, 4, (4, 3))),
+    "pair_matrix_cores": lt.layer(lt.parallel(lt.left(4, 2, 32, 64, 3, temp=(0.3, 16)), lt.right(2, 1, 72, 40, 3, 8, 8), 0.75, 0.5), None),
+    "experts": lt.layer(lt.keyed(1, 1, 8, rot=4), lt.moe(20, 9, 4, (3, 2))),
     "experts_plain_top": lt.layer(lt.keyed(1, 1, 8), lt.moe(12, 5, 2)),
 }
 
@@ -520,7 +523,7 @@ def random_config(rng: random.Random) -> dict:
     config = {"architecture": "Legavik", "vocab": rng.choice([50, 97, 256]), "width": width,
               "norm": {"eps": rng.choice([1e-6, 1e-5])}, "layers": layers}
     if rng.random() < 0.7:
-        config["logit_softcap"] = rng.choice([1.5, 10.0, 30.0])
+        config["logit_softcap"] = rng.choice([1.5, 10.0, 40.0])
     return config
 
 

@@ -18,7 +18,7 @@
 // of the run's type, or `splits` 32-bit partial sums, of which the columns named by *_at are read.
 #include "common.hpp"
 
-#define DS_MAX_LOW 128
+#define DS_MAX_LOW 256
 
 template <typename P>
 __device__ __forceinline__ float ds_input(const P* p, int splits, size_t stride) {

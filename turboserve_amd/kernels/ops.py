@@ -1047,12 +1047,12 @@ class Ops:
         _need(u.dtype == torch.float32 and u.is_contiguous() and u.shape == (tokens, 2 * keys + values),
               "the convolved q | k | v must be float32 [T, 2 G D + H Dv]")
         _need(heads % kv_heads == 0 and 1 <= head_dim <= 256, "heads in equal shares of the key heads, up to 256 key channels")
-        _need(a2.dim() == 2 and a2.shape[0] == heads * head_dim and 1 <= a2.shape[1] <= 128 and a2.dtype == dtype and a2.is_contiguous()
+        _need(a2.dim() == 2 and a2.shape[0] == heads * head_dim and 1 <= a2.shape[1] <= 256 and a2.dtype == dtype and a2.is_contiguous()
               and dt_bias.shape == (heads * head_dim,) and dt_bias.dtype == dtype and dt_bias.is_contiguous(),
-              "the decay's matrix must be [H D, R] with R up to 128 and its bias [H D], of the run dtype")
-        _need(g2.dim() == 2 and g2.shape[0] == values and 1 <= g2.shape[1] <= 128 and g2.dtype == dtype and g2.is_contiguous()
+              "the decay's matrix must be [H D, R] with R up to 256 and its bias [H D], of the run dtype")
+        _need(g2.dim() == 2 and g2.shape[0] == values and 1 <= g2.shape[1] <= 256 and g2.dtype == dtype and g2.is_contiguous()
               and gain.shape == (value_dim,) and gain.dtype == dtype and gain.is_contiguous(),
-              "the gate's matrix must be [H Dv, R] with R up to 128 and the gain [Dv], of the run dtype")
+              "the gate's matrix must be [H Dv, R] with R up to 256 and the gain [Dv], of the run dtype")
         _need(a_log.shape == (heads,) and a_log.dtype == torch.float32 and a_log.is_contiguous(), "a_log must be float32 [H]")
         _need(state.dtype == torch.float32 and state.is_contiguous() and state.shape[1:] == (heads, head_dim, value_dim),
               "the state must be float32 [slots, H, D, Dv]")

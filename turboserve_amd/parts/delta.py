@@ -53,8 +53,8 @@ class GatedDeltaRule(Mixer):
         if not 1 <= self.taps <= 8:
             raise ValueError(f"{where}: a convolution of {self.taps} taps is outside 1..8")
         for rank in (self.decay_rank, self.gate_rank):
-            if rank is not None and not 1 <= rank <= 128:
-                raise ValueError(f"{where}: a low-rank input of {rank} is outside 1..128")
+            if rank is not None and not 1 <= rank <= 256:
+                raise ValueError(f"{where}: a low-rank input of {rank} is outside 1..256")
         self.names = {"q": "q", "k": "k", "v": "v", "beta": "b", "a1": "a1", "a2": "a2", "dt": "dt_bias", "a_log": "A_log",
                       "g1": "g1", "g2": "g2", "norm": "norm", "o": "o", **(names or {})}
         self.conv_suffix = conv_suffix
@@ -105,9 +105,9 @@ class GatedDeltaRule(Mixer):
         self.a2 = tensors[self.name(n["a2"])].contiguous()
         self.g2 = tensors[self.name(n["g2"])].contiguous()
         for low, high, what in ((a1, self.a2, "decay"), (g1, self.g2, "gate")):
-            if low.shape[0] != high.shape[1] or not 1 <= low.shape[0] <= 128:
+            if low.shape[0] != high.shape[1] or not 1 <= low.shape[0] <= 256:
                 raise ValueError(f"{self.prefix}: the {what}'s two matrices meet at {low.shape[0]} and {high.shape[1]} "
-                                 "elements; they must agree and be 1..128")
+                                 "elements; they must agree and be 1..256")
         self.beta_at = self.channels
         self.decay_at = self.beta_at + self.num_heads
         self.gate_at = self.decay_at + int(a1.shape[0])

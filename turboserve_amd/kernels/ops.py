@@ -992,8 +992,9 @@ class Ops:
         """A short causal convolution over time on the ``C`` columns of ``proj`` from ``first_col`` on (``taps [C,
         K]``: ``y_t = sum_j taps[:, j] u_(t - K + 1 + j)``), continuing every request from the ``K - 1`` inputs its
         state slot holds (``state [slots, max(K - 1, 1), C]`` 32-bit, oldest first) and leaving its last ``K - 1``
-        inputs there.  ``proj`` is ``[T, W]`` of the run dtype or 32-bit partial sums.  Returns ``[T, C]`` of the
-        run dtype (32-bit with ``out_float32``), through ``silu`` if asked."""
+        inputs there (by a second launch; in a step whose requests all bring one token the first launch does it).
+        ``proj`` is ``[T, W]`` of the run dtype or 32-bit partial sums.  Returns ``[T, C]`` of the run dtype (32-bit
+        with ``out_float32``), through ``silu`` if asked."""
         _gpu(proj, taps, state, state_slots, token_seq, query_start_loc)
         _i32(state_slots, "state_slots")
         _i32(token_seq, "token_seq")

@@ -10,7 +10,8 @@
 //   ts_delta_scan     per (request, head, 8 or 32 value columns): the request's tokens in order, the state
 //                     from and to the request's slot;
 //   ts_delta_finish   per (token, head): o divided by its root mean square, times a gain [Dv] shared by
-//                     the heads, times sigmoid(g2 . low'), rounded once to the run's type.
+//                     the heads, times sigmoid(g2 . low') (and a scale), rounded once to the run's type; its
+//                     rows may be a part of a wider buffer's.
 // Of the two low-rank matrices a2 [H D, R] and g2 [H Dv, R'] a lane walks its channel's row; over a prompt a
 // wavefront of the launches around the walk takes eight tokens, so that it reads its rows once for all eight (in a
 // step of few tokens: one token each).
@@ -299,7 +300,7 @@ template <typename T, typename P, int DS_TOKENS>
 __global__ void __launch_bounds__(64 * DS_ITEMS)
 delta_finish_kernel(T* __restrict__ y, const float* __restrict__ o, const P* __restrict__ proj, int splits, size_t split_stride,
                     int width, int low_at, int low, const T* __restrict__ g2, const T* __restrict__ gain, float eps, int tokens,
-                    int heads, int vdim) {
+                    int heads, int vdim, float scale, size_t out_stride) {
   __shared__ __attribute__((aligned(16))) float lows_of[DS_ITEMS][DS_MAX_LOW][DS_TOKENS];
   const int wave = threadIdx.x / TS_WAVE, lane = threadIdx.x % TS_WAVE;
   const int tiles = (tokens + DS_TOKENS - 1) / DS_TOKENS;
@@ -339,7 +340,7 @@ delta_finish_kernel(T* __restrict__ y, const float* __restrict__ o, const P* __r
     for (int tt = 0; tt < DS_TOKENS; ++tt) {
       if (tt < count) {
         const size_t at = ((size_t)(t0 + tt) * heads + h) * vdim + c;
-        y[at] = from_float<T>(o[at] * by[tt] * g / (1.f + expf(-z[tt])));
+        y[(size_t)(t0 + tt) * out_stride + (size_t)h * vdim + c] = from_float<T>(scale * o[at] * by[tt] * g / (1.f + expf(-z[tt])));
       }
     }
   }
@@ -405,9 +406,9 @@ extern "C" int ts_delta_scan(float* o, float* state, const float* qn, const floa
 
 extern "C" int ts_delta_finish(void* y, const float* o, const void* proj, int in_f32, int splits, long split_stride, int width,
                                int low_at, int low, const void* g2, const void* gain, float eps, int tokens, int heads, int vdim,
-                               int dtype, hipStream_t stream) {
+                               int dtype, float scale, long out_stride, hipStream_t stream) {
   if (tokens == 0) return TS_OK;
-  if (!y || !o || !proj || !g2 || !gain) return TS_ERR_ARG;
+  if (!y || !o || !proj || !g2 || !gain || out_stride < (long)heads * vdim) return TS_ERR_ARG;
   if (heads < 1 || heads > 65535 || vdim < 1 || low < 1 || low > DS_MAX_LOW || splits < 1 || low_at < 0 || low_at + low > width)
     return TS_ERR_SHAPE;
   const int per = tokens >= 64 ? 8 : 1;
@@ -416,10 +417,10 @@ extern "C" int ts_delta_finish(void* y, const float* o, const void* proj, int in
 #define DS_GO(T, P)                                                                                                   \
   if (per == 8)                                                                                                       \
     hipLaunchKernelGGL((delta_finish_kernel<T, P, 8>), grid, block, 0, stream, (T*)y, o, (const P*)proj, splits,       \
-                       (size_t)split_stride, width, low_at, low, (const T*)g2, (const T*)gain, eps, tokens, heads, vdim); \
+                       (size_t)split_stride, width, low_at, low, (const T*)g2, (const T*)gain, eps, tokens, heads, vdim, scale, (size_t)out_stride); \
   else                                                                                                                \
     hipLaunchKernelGGL((delta_finish_kernel<T, P, 1>), grid, block, 0, stream, (T*)y, o, (const P*)proj, splits,       \
-                       (size_t)split_stride, width, low_at, low, (const T*)g2, (const T*)gain, eps, tokens, heads, vdim)
+                       (size_t)split_stride, width, low_at, low, (const T*)g2, (const T*)gain, eps, tokens, heads, vdim, scale, (size_t)out_stride)
   if (dtype == TS_F32) DS_GO(float, float);
   else if (dtype == TS_BF16 && in_f32) DS_GO(bf16_t, float);
   else if (dtype == TS_BF16) DS_GO(bf16_t, bf16_t);

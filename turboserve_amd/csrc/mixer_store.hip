@@ -238,12 +238,12 @@ __device__ __forceinline__ float4 gate_values4<bf16_t>(const bf16_t* at) {
 template <typename T, typename P, typename V>
 __global__ void __launch_bounds__(256)
 head_gate_kernel(T* __restrict__ out, const V* __restrict__ values, const P* __restrict__ proj, int splits,
-                 size_t split_stride, int width, int gate_at, int heads, int vdim) {
+                 size_t split_stride, int width, int gate_at, int heads, int vdim, float scale, size_t out_stride) {
   const int t = blockIdx.x;
   const int per = heads * vdim;
   for (int i = blockIdx.y * blockDim.x + threadIdx.x; i < per; i += gridDim.y * blockDim.x) {
     const float g = folded(proj + (size_t)t * width + gate_at + i / vdim, splits, split_stride);
-    out[(size_t)t * per + i] = from_float<T>(to_float(values[(size_t)t * per + i]) / (1.f + expf(-g)));
+    out[(size_t)t * out_stride + i] = from_float<T>(scale * to_float(values[(size_t)t * per + i]) / (1.f + expf(-g)));
   }
 }
 
@@ -251,15 +251,15 @@ head_gate_kernel(T* __restrict__ out, const V* __restrict__ values, const P* __r
 template <typename T, typename P, typename V>
 __global__ void __launch_bounds__(256)
 head_gate_vec4_kernel(T* __restrict__ out, const V* __restrict__ values, const P* __restrict__ proj, int splits,
-                      size_t split_stride, int width, int gate_at, int heads, int vdim) {
+                      size_t split_stride, int width, int gate_at, int heads, int vdim, float scale, size_t out_stride) {
   const int t = blockIdx.x;
   const int per = heads * vdim;
   const int i = 4 * (blockIdx.y * blockDim.x + threadIdx.x);
   if (i >= per) return;
   const float4 v = gate_values4<V>(values + (size_t)t * per + i);
   const float g = folded(proj + (size_t)t * width + gate_at + i / vdim, splits, split_stride);
-  const float d = 1.f + expf(-g);
-  T* to = out + (size_t)t * per + i;
+  const float d = (1.f + expf(-g)) / scale;
+  T* to = out + (size_t)t * out_stride + i;
   if constexpr (std::is_same<T, float>::value) {
     *reinterpret_cast<float4*>(to) = make_float4(v.x / d, v.y / d, v.z / d, v.w / d);
   } else {
@@ -272,36 +272,38 @@ head_gate_vec4_kernel(T* __restrict__ out, const V* __restrict__ values, const P
 
 template <typename T, typename P, typename V>
 static void launch_head_gate(void* out, const void* values, const void* proj, int splits, size_t split_stride, int tokens,
-                             int width, int gate_at, int heads, int vdim, hipStream_t stream) {
+                             int width, int gate_at, int heads, int vdim, float scale, size_t out_stride, hipStream_t stream) {
   const int per = heads * vdim;
-  if (vdim % 4 == 0 && ((uintptr_t)out | (uintptr_t)values) % 16 == 0) {
+  if (vdim % 4 == 0 && ((uintptr_t)out | (uintptr_t)values) % 16 == 0 && out_stride % 4 == 0 && scale != 0.f) {
     const dim3 grid(tokens, (per / 4 + 255) / 256);
     hipLaunchKernelGGL((head_gate_vec4_kernel<T, P, V>), grid, dim3(256), 0, stream, (T*)out, (const V*)values, (const P*)proj,
-                       splits, split_stride, width, gate_at, heads, vdim);
+                       splits, split_stride, width, gate_at, heads, vdim, scale, out_stride);
   } else {
     const dim3 grid(tokens, (per + 1023) / 1024);
     hipLaunchKernelGGL((head_gate_kernel<T, P, V>), grid, dim3(256), 0, stream, (T*)out, (const V*)values, (const P*)proj,
-                       splits, split_stride, width, gate_at, heads, vdim);
+                       splits, split_stride, width, gate_at, heads, vdim, scale, out_stride);
   }
 }
 
-// values_f32: the values are 32-bit (else of the run's type, as the attention kernels leave them).
+// values_f32: the values are 32-bit (else of the run's type, as the attention kernels leave them).  The result
+// is multiplied by `scale` as well, and its rows lie `out_stride` elements apart (a part of a wider buffer).
 extern "C" int ts_head_gate(void* out, const void* values, int values_f32, const void* proj, int in_f32, int splits,
                             long split_stride, int tokens, int width, int gate_at, int heads, int vdim, int dtype,
-                            hipStream_t stream) {
+                            float scale, long out_stride, hipStream_t stream) {
   if (tokens == 0) return TS_OK;
-  if (!out || !values || !proj || heads < 1 || vdim < 1 || splits < 1 || gate_at < 0 || gate_at + heads > width)
+  if (!out || !values || !proj || heads < 1 || vdim < 1 || splits < 1 || gate_at < 0 || gate_at + heads > width ||
+      out_stride < (long)heads * vdim)
     return TS_ERR_ARG;
   if (dtype == TS_F32)
-    launch_head_gate<float, float, float>(out, values, proj, splits, (size_t)split_stride, tokens, width, gate_at, heads, vdim, stream);
+    launch_head_gate<float, float, float>(out, values, proj, splits, (size_t)split_stride, tokens, width, gate_at, heads, vdim, scale, (size_t)out_stride, stream);
   else if (dtype == TS_BF16 && in_f32 && values_f32)
-    launch_head_gate<bf16_t, float, float>(out, values, proj, splits, (size_t)split_stride, tokens, width, gate_at, heads, vdim, stream);
+    launch_head_gate<bf16_t, float, float>(out, values, proj, splits, (size_t)split_stride, tokens, width, gate_at, heads, vdim, scale, (size_t)out_stride, stream);
   else if (dtype == TS_BF16 && in_f32)
-    launch_head_gate<bf16_t, float, bf16_t>(out, values, proj, splits, (size_t)split_stride, tokens, width, gate_at, heads, vdim, stream);
+    launch_head_gate<bf16_t, float, bf16_t>(out, values, proj, splits, (size_t)split_stride, tokens, width, gate_at, heads, vdim, scale, (size_t)out_stride, stream);
   else if (dtype == TS_BF16 && values_f32)
-    launch_head_gate<bf16_t, bf16_t, float>(out, values, proj, 1, (size_t)0, tokens, width, gate_at, heads, vdim, stream);
+    launch_head_gate<bf16_t, bf16_t, float>(out, values, proj, 1, (size_t)0, tokens, width, gate_at, heads, vdim, scale, (size_t)out_stride, stream);
   else if (dtype == TS_BF16)
-    launch_head_gate<bf16_t, bf16_t, bf16_t>(out, values, proj, 1, (size_t)0, tokens, width, gate_at, heads, vdim, stream);
+    launch_head_gate<bf16_t, bf16_t, bf16_t>(out, values, proj, 1, (size_t)0, tokens, width, gate_at, heads, vdim, scale, (size_t)out_stride, stream);
   else
     return TS_ERR_DTYPE;
   return ts_launch_status();

@@ -87,7 +87,7 @@ _SIGNATURES: dict[str, dict[str, list]] = {
                             c_void_p, c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_int, c_int, c_int, c_int, c_int, c_int,
                             c_void_p],
         "ts_head_gate": [c_void_p, c_void_p, c_int, c_void_p, c_int, c_int, c_long, c_int, c_int, c_int, c_int, c_int, c_int,
-                         c_void_p],
+                         c_float, c_long, c_void_p],
         "ts_scaled_pair": [c_void_p, c_void_p, c_int, c_int, c_long, c_float, c_void_p, c_int, c_int, c_long, c_float, c_long,
                            c_int, c_void_p],
         "ts_add_tanh_norm": [c_void_p, c_void_p, c_void_p, c_int, c_int, c_long, c_void_p, c_void_p, c_float, c_void_p, c_int,
@@ -102,7 +102,7 @@ _SIGNATURES: dict[str, dict[str, list]] = {
         "ts_delta_scan": [c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_int,
                           c_int, c_int, c_int, c_int, c_int, c_int, c_void_p],
         "ts_delta_finish": [c_void_p, c_void_p, c_void_p, c_int, c_int, c_long, c_int, c_int, c_int, c_void_p, c_void_p,
-                            c_float, c_int, c_int, c_int, c_int, c_void_p],
+                            c_float, c_int, c_int, c_int, c_int, c_float, c_long, c_void_p],
         "ts_stream_fold": [c_void_p, c_void_p, c_int, c_int, c_long, c_long, c_int, c_int, c_void_p],
         "ts_stream_pair": [c_void_p, c_void_p, c_void_p, c_int, c_int, c_int, c_void_p],
         "ts_linear_state_scan": [c_void_p, c_void_p, c_int, c_int, c_long, c_void_p, c_void_p, c_float, c_void_p, c_void_p,
@@ -814,20 +814,36 @@ class Ops:
             block_size, 1 if neighbours else 0, int(tail), dtype_code(run_dtype), self.stream()), "ts_latent_store")
         return q_plain, q_wide
 
-    def head_gate(self, values: torch.Tensor, proj: torch.Tensor, gate_at: int, heads: int, dtype: torch.dtype) -> torch.Tensor:
+    def _columns_of(self, out: tuple[torch.Tensor, int] | None, tokens: int, width: int, dtype: torch.dtype, device):
+        """Where a kernel writes ``[tokens, width]`` of ``dtype``: a buffer of its own, or the columns ``col0 .. col0 +
+        width - 1`` of a wider ``[tokens, W]`` buffer handed in as ``(buffer, col0)``.  Returns ``(result, pointer, row
+        stride)``."""
+        if out is None:
+            made = self.rows_buffer(tokens, width, dtype, device)
+            return made, _ptr(made), width
+        buffer, col0 = out
+        _gpu(buffer)
+        _need(buffer.dim() == 2 and buffer.is_contiguous() and buffer.dtype == dtype and buffer.shape[0] == tokens
+              and 0 <= col0 and col0 + width <= buffer.shape[1], "the columns must lie inside a contiguous [T, W] buffer of the run dtype")
+        return buffer, buffer.data_ptr() + col0 * buffer.element_size(), buffer.shape[1]
+
+    def head_gate(self, values: torch.Tensor, proj: torch.Tensor, gate_at: int, heads: int, dtype: torch.dtype, *,
+                  scale: float = 1.0, out: tuple[torch.Tensor, int] | None = None) -> torch.Tensor:
         """``[T, H Dv]`` of ``dtype``: head ``h``'s ``Dv`` elements of ``values [T, H Dv]`` (32-bit, or of ``dtype``) times
         ``sigmoid`` of column ``gate_at + h`` of the token's row of ``proj`` (a projection of the run
-        dtype or its 32-bit partial sums), in 32-bit with one rounding."""
+        dtype or its 32-bit partial sums) and times ``scale``, in 32-bit with one rounding.  ``out = (buffer, col0)``:
+        the result is written into those columns of a wider buffer, which is returned."""
         _gpu(values, proj)
         tokens, width = proj.shape[-2], proj.shape[-1]
         is_f32, splits, stride = self._partials(proj, tokens, width, dtype, "projection")
         _need(values.dtype in (torch.float32, dtype) and values.is_contiguous() and values.dim() == 2 and values.shape[0] == tokens
               and values.shape[1] % heads == 0 and 0 <= gate_at and gate_at + heads <= width,
               "values must be [T, H Dv], 32-bit or of the run dtype, and the gates' columns inside the projection")
-        out = self.rows_buffer(tokens, values.shape[1], dtype, values.device)
-        _check(self.core.ts_head_gate(_ptr(out), _ptr(values), 1 if values.dtype == torch.float32 else 0, _ptr(proj), is_f32, splits, stride, tokens, width, gate_at,
-                                      heads, values.shape[1] // heads, dtype_code(dtype), self.stream()), "ts_head_gate")
-        return out
+        result, pointer, out_stride = self._columns_of(out, tokens, values.shape[1], dtype, values.device)
+        _check(self.core.ts_head_gate(pointer, _ptr(values), 1 if values.dtype == torch.float32 else 0, _ptr(proj), is_f32, splits,
+                                      stride, tokens, width, gate_at, heads, values.shape[1] // heads, dtype_code(dtype),
+                                      float(scale), out_stride, self.stream()), "ts_head_gate")
+        return result
 
     def stream_fold(self, residual: torch.Tensor, part: torch.Tensor, dtype: torch.dtype, *, assign: bool = False) -> None:
         """``residual [T, H] += part`` in 32-bit, in place (``assign``: ``residual = part``); ``part`` is a
@@ -1028,7 +1044,7 @@ class Ops:
                    dt_bias: torch.Tensor, a_log: torch.Tensor, g2: torch.Tensor, gain: torch.Tensor, eps: float,
                    state: torch.Tensor, state_slots: torch.Tensor, query_start_loc: torch.Tensor, tokens: int, num_seqs: int,
                    heads: int, kv_heads: int, head_dim: int, value_dim: int, dtype: torch.dtype,
-                   num_long_seqs: int = 0) -> torch.Tensor:
+                   num_long_seqs: int = 0, scale: float = 1.0, out: tuple[torch.Tensor, int] | None = None) -> torch.Tensor:
         """The gated delta rule over a step: per head and request a 32-bit state ``S [D, Dv]`` (``state [slots, H,
         D, Dv]``) that every token decays, corrects and reads: ``S <- diag(g) S; w = beta (v - S^T k); S <- S + k
         w^T; o = S^T q``.  ``u [T, 2 G D + H Dv]`` (32-bit) holds the step's convolved ``q | k | v``; ``q`` and ``k``
@@ -1038,7 +1054,8 @@ class Ops:
         by ``gain [Dv]`` and by ``sigmoid(g2 . low')``, ``low'`` the ``g2.shape[1]`` columns from ``gate_at`` on.
         The first ``num_long_seqs`` requests (those that bring several tokens) are walked with the state spread
         thinly over many workgroups, the others with whole cache lines of the state a workgroup.  Returns ``[T, H
-        Dv]`` of ``dtype``."""
+        Dv]`` of ``dtype``, times ``scale``; with ``out = (buffer, col0)`` written into those columns of a wider buffer,
+        which is returned."""
         _gpu(u, proj, a2, dt_bias, a_log, g2, gain, state, state_slots, query_start_loc)
         _i32(state_slots, "state_slots")
         _i32(query_start_loc, "query_start_loc")
@@ -1072,9 +1089,10 @@ class Ops:
             _check(self.core.ts_delta_scan(_ptr(o), _ptr(state), _ptr(qn), _ptr(kn), _ptr(kq), _ptr(decay), _ptr(beta), _ptr(u),
                                            _ptr(state_slots), _ptr(query_start_loc), first, count, heads, kv_heads, head_dim,
                                            value_dim, spread, self.stream()), "ts_delta_scan")
-        y = self.rows_buffer(tokens, values, dtype, device)
-        _check(self.core.ts_delta_finish(_ptr(y), _ptr(o), _ptr(proj), is_f32, splits, stride, width, gate_at, g2.shape[1], _ptr(g2),
-                                         _ptr(gain), float(eps), tokens, heads, value_dim, code, self.stream()), "ts_delta_finish")
+        y, pointer, out_stride = self._columns_of(out, tokens, values, dtype, device)
+        _check(self.core.ts_delta_finish(pointer, _ptr(o), _ptr(proj), is_f32, splits, stride, width, gate_at, g2.shape[1], _ptr(g2),
+                                         _ptr(gain), float(eps), tokens, heads, value_dim, code, float(scale), out_stride,
+                                         self.stream()), "ts_delta_finish")
         return y
 
     # -- routed feed-forward --------------------------------------------------------------------

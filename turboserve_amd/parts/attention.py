@@ -256,6 +256,22 @@ class GroupedQueryAttention(Mixer):
         self.position.load(tensors)
 
     def forward(self, x: torch.Tensor, ctx, cache) -> torch.Tensor:
+        return self.runtime.ops.linear(self.heads_out(x, ctx, cache), self.o_weight, self.o_bias_tensor, for_residual=True)
+
+    @property
+    def out_features(self) -> int:
+        """The width of what the output matrix multiplies."""
+        return self.out_size
+
+    def scales_its_heads(self) -> bool:
+        """Whether :meth:`heads_out` can apply a scale and write into a wider buffer (the gate's launch does both)."""
+        return self.gate_name is not None
+
+    def heads_out(self, x: torch.Tensor, ctx, cache, *, scale: float = 1.0, out: tuple | None = None) -> torch.Tensor:
+        """Everything but the output matrix: ``[T, Hq Dv]`` of the run dtype, what that matrix multiplies.  With a gate
+        per head the result may be multiplied by ``scale`` and written into columns of a wider buffer (``out =
+        (buffer, col0)``): a caller that adds this mixer's output to another's can then run both output matrices as
+        one product."""
         ops = self.runtime.ops
         qkv = proj = ops.linear(x, self.qkv_weight, self.qkv_bias_tensor)
         more, shape = {}, {}
@@ -296,8 +312,11 @@ class GroupedQueryAttention(Mixer):
         attended = self.attend(q, q_stride, ctx, cache)
         if self.gate_name is not None:
             # Every head's output times the sigmoid of its gate (the projection's last columns), rounded once.
-            attended = ops.head_gate(attended, proj, self.q_size + self.kv_size + self.v_size, self.num_heads, self.runtime.dtype)
-        return ops.linear(attended, self.o_weight, self.o_bias_tensor, for_residual=True)
+            return ops.head_gate(attended, proj, self.q_size + self.kv_size + self.v_size, self.num_heads, self.runtime.dtype,
+                                 scale=scale, out=out)
+        if scale != 1.0 or out is not None:
+            raise ValueError(f"{self.prefix}: without a gate per head nothing scales or places the heads' output")
+        return attended
 
     def attend(self, qkv: torch.Tensor, q_stride: int, ctx, cache: PagedKVView) -> torch.Tensor:
         """``[T, Hq D]`` attention output for the step's encoded queries: the first ``Hq D``

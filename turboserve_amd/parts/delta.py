@@ -120,15 +120,29 @@ class GatedDeltaRule(Mixer):
         self.o_weight = tensors[self.name(n["o"])].contiguous()
 
     def forward(self, x: torch.Tensor, ctx, cache) -> torch.Tensor:
+        return self.runtime.ops.linear(self.heads_out(x, ctx, cache), self.o_weight, for_residual=True)
+
+    o_bias_tensor = None
+
+    @property
+    def out_features(self) -> int:
+        """The width of what the output matrix multiplies."""
+        return self.value_size
+
+    def scales_its_heads(self) -> bool:
+        return True
+
+    def heads_out(self, x: torch.Tensor, ctx, cache, *, scale: float = 1.0, out: tuple | None = None) -> torch.Tensor:
+        """Everything but the output matrix: ``[T, H Dv]`` of the run dtype times ``scale``, optionally written into
+        columns of a wider buffer (``out = (buffer, col0)``)."""
         ops, dtype = self.runtime.ops, self.runtime.dtype
         memory, held = cache
         proj = ops.linear(x, self.fused)
         u = ops.short_conv(proj, 0, self.conv_weight, held.state, ctx.state_slots, ctx.token_seq, ctx.query_start_loc,
                            tokens=ctx.num_tokens, num_seqs=ctx.num_seqs, dtype=dtype, silu=True, out_float32=True)
-        y = ops.delta_rule(u, proj, beta_at=self.beta_at, decay_at=self.decay_at, gate_at=self.gate_at, a2=self.a2,
-                           dt_bias=self.dt, a_log=self.a_log, g2=self.g2, gain=self.gain, eps=self.norm_eps,
-                           state=memory.state, state_slots=ctx.state_slots, query_start_loc=ctx.query_start_loc,
-                           tokens=ctx.num_tokens, num_seqs=ctx.num_seqs, heads=self.num_heads, kv_heads=self.num_kv_heads,
-                           head_dim=self.head_dim, value_dim=self.value_dim, dtype=dtype,
-                           num_long_seqs=0 if ctx.recorded else ctx.num_prefill_seqs)
-        return ops.linear(y, self.o_weight, for_residual=True)
+        return ops.delta_rule(u, proj, beta_at=self.beta_at, decay_at=self.decay_at, gate_at=self.gate_at, a2=self.a2,
+                              dt_bias=self.dt, a_log=self.a_log, g2=self.g2, gain=self.gain, eps=self.norm_eps,
+                              state=memory.state, state_slots=ctx.state_slots, query_start_loc=ctx.query_start_loc,
+                              tokens=ctx.num_tokens, num_seqs=ctx.num_seqs, heads=self.num_heads, kv_heads=self.num_kv_heads,
+                              head_dim=self.head_dim, value_dim=self.value_dim, dtype=dtype,
+                              num_long_seqs=0 if ctx.recorded else ctx.num_prefill_seqs, scale=scale, out=out)

@@ -159,6 +159,38 @@ def test_the_short_convolution_carries_its_last_inputs(ops, dtype, taps, channel
     assert torch.isnan(state[[1, 4]]).all() if taps > 1 else True
 
 
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+def test_the_weighted_sum_of_two_outputs(ops, dtype):
+    """Two parts' outputs, each a tensor of the run's type or partial sums, as one 32-bit addend."""
+    g = torch.Generator().manual_seed(3)
+    dense, sums = torch.randn(7, 52, generator=g).to(dtype), torch.randn(3, 7, 52, generator=g)
+    other = torch.randn(7, 52, generator=g).to(dtype)
+    got = ops.scaled_pair(dense.to(DEV), 0.6, sums.to(DEV), -1.3, dtype)
+    assert got.shape == (1, 7, 52) and got.dtype == torch.float32
+    near(got[0], 0.6 * dense.float() - 1.3 * sums.sum(0), torch.float32)
+    near(ops.scaled_pair(sums.to(DEV), 2.0, sums.to(DEV), 0.5, dtype)[0], 2.5 * sums.sum(0), torch.float32)
+    near(ops.scaled_pair(dense.to(DEV), 1.0, other.to(DEV), 1.0, dtype)[0], dense.float() + other.float(), torch.float32)
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+@pytest.mark.parametrize("heads,vdim,col0,scale", [(3, 12, 8, 0.6), (1, 20, 0, -0.8), (8, 64, 16, 1.0), (5, 7, 3, 0.0)])
+def test_a_gate_per_head_scales_and_places_its_result(ops, dtype, heads, vdim, col0, scale):
+    """The gate's launch multiplies by a weight as well and writes into columns of a wider buffer, whose other
+    columns stay as they are; values of the run's own type and 32-bit ones."""
+    g = torch.Generator().manual_seed(heads * 10 + vdim)
+    tokens, width = 9, heads + 5
+    proj = torch.randn(tokens, width, generator=g).to(dtype)
+    for values in (torch.randn(tokens, heads * vdim, generator=g), torch.randn(tokens, heads * vdim, generator=g).to(dtype)):
+        gate = torch.sigmoid(proj.float()[:, 2:2 + heads]).repeat_interleave(vdim, dim=1)
+        want = scale * values.float() * gate
+        wide = torch.full((tokens, col0 + heads * vdim + 4), 7.0, dtype=dtype, device=DEV)
+        got = ops.head_gate(values.to(DEV), proj.to(DEV), 2, heads, dtype, scale=scale, out=(wide, col0))
+        assert got is wide
+        near(wide[:, col0:col0 + heads * vdim], want, dtype)
+        assert bool((wide[:, :col0] == 7.0).all()) and bool((wide[:, col0 + heads * vdim:] == 7.0).all())
+        near(ops.head_gate(values.to(DEV), proj.to(DEV), 2, heads, dtype), values.float() * gate, dtype)
+
+
 def delta_inputs(g, tokens, heads, kv_heads, dim, vdim, low_a, low_g, dtype):
     keys, values = kv_heads * dim, heads * vdim
     u = torch.randn(tokens, 2 * keys + values, generator=g)
